@@ -1,0 +1,136 @@
+/*
+ * tftq -- FP8 (OCP e4m3fn) quantized-collective kernels for AMD MI355X (gfx950).
+ *
+ * C ABI of libtftq.so.  Plain pointers and sizes only; no torch types.
+ * The three compute entry points replace the three launchers of the reference
+ * (torchft/quantization.py): fused_quantize_into_fp8 (:531-588),
+ * fused_reduce_fp8 (:638-686) and fused_dequantize_from_fp8 (:591-635).
+ * The plan replaces _prepare_quantize_fp8 (:431-528).
+ *
+ * Conventions
+ *  - every function returns 0 on success; a negative value is a TFTQ_E_* code,
+ *    a positive value is a hipError_t.  Nothing aborts or throws.
+ *  - device pointers must belong to the device that is current on the calling
+ *    thread; kernels are enqueued on `stream` (a hipStream_t passed as void*,
+ *    NULL = the null stream) and the host is never synchronised.
+ *  - functions are thread-safe; a plan may be used from several threads at
+ *    once (it is immutable after tftq_plan_set_device_table).
+ *
+ * Packed buffer (byte-for-byte the reference's, quantization.py:108-123,
+ * 495-503), for tensor i of shape [m_i, n_i] and group size ws:
+ *    row_bytes_i  = (ceil(n_i / 4) + 1) * 4
+ *    slice_rows_i = ceil(m_i / ws)
+ *    slot_off_i   = sum_{j<i} slice_rows_j * row_bytes_j
+ *    slot_size    = sum_i slice_rows_i * row_bytes_i
+ *    output_size  = ws * slot_size
+ *    addr(i, r)   = (r / slice_rows_i) * slot_size + slot_off_i
+ *                   + (r % slice_rows_i) * row_bytes_i
+ *    at addr: [fp32 scale][n_i e4m3fn codes][zero padding to row_bytes_i]
+ */
+#ifndef TFTQ_H
+#define TFTQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TFTQ_VERSION 1
+
+/* element types of the tensors being (de)quantized (quantization.py:474-478) */
+#define TFTQ_F32 0
+#define TFTQ_F16 1
+#define TFTQ_BF16 2
+
+/* error codes (negative); positive return values are hipError_t */
+#define TFTQ_E_ARG (-1)      /* bad argument (null pointer, ws <= 0, rank out of range ...) */
+#define TFTQ_E_DTYPE (-2)    /* "Only fp32, fp16 and bf16 are supported" (:474-478) */
+#define TFTQ_E_SHAPE (-3)    /* negative or too large dimension */
+#define TFTQ_E_SIZE (-4)     /* "Output size does not match" (:621, :672) */
+#define TFTQ_E_NOMEM (-5)    /* host allocation failed */
+#define TFTQ_E_NOTABLE (-6)  /* plan needs a device table that was not provided */
+#define TFTQ_E_ARCH (-7)     /* current device is not gfx950 */
+
+typedef struct tftq_plan tftq_plan;
+
+/* library version (TFTQ_VERSION of the build) */
+int tftq_version(void);
+
+/* Text for a return value of this library (static storage). */
+const char *tftq_strerror(int code);
+
+/* 0 when the current device can run the kernels (gfx950), else TFTQ_E_ARCH or
+ * a hipError_t. */
+int tftq_check_device(void);
+
+/*
+ * Layout arithmetic of _prepare_quantize_fp8 (quantization.py:486-503), host
+ * only.  shapes: [n_tensors][2] = (m, n); 1-D tensors are passed as (k, 1)
+ * (:487-488).  slot_off (may be NULL) receives n_tensors byte offsets.
+ */
+int tftq_layout(int n_tensors, const int64_t *shapes, int ws, int64_t *slot_off,
+                int64_t *slot_size, int64_t *output_size);
+
+/*
+ * Builds the work plan for one list of tensors: the layout above plus the
+ * partition of all rows into workgroups for the three kernels.  Replaces the
+ * four device tables that _prepare_quantize_fp8 uploads on every call
+ * (quantization.py:505-515).  Host only, no HIP call.
+ *   dtype    TFTQ_F32 / TFTQ_F16 / TFTQ_BF16
+ *   ptrs     [n_tensors] device address of element (0,0) of each tensor; may
+ *            be NULL for a plan that is only used with tftq_reduce
+ *   shapes   [n_tensors][2] (m, n)
+ *   strides  [n_tensors][2] element strides (row, column); any values
+ */
+int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
+                     const int64_t *shapes, const int64_t *strides, int ws,
+                     tftq_plan **out);
+void tftq_plan_destroy(tftq_plan *plan);
+
+int64_t tftq_plan_output_size(const tftq_plan *plan); /* bytes of the packed buffer */
+int64_t tftq_plan_slot_size(const tftq_plan *plan);   /* output_size / ws */
+int64_t tftq_plan_max_rows(const tftq_plan *plan);    /* i_max_row_num of the reference */
+
+/*
+ * Plans with few tensors carry their descriptors in the kernel arguments and
+ * need no device memory: tftq_plan_table_bytes() returns 0.  Larger plans need
+ * a device copy of the descriptor table: allocate tftq_plan_table_bytes()
+ * bytes (256-byte aligned) on the device, copy tftq_plan_table_host() into it
+ * and hand the address over with tftq_plan_set_device_table() before the first
+ * compute call.  The library never allocates device memory.
+ */
+int64_t tftq_plan_table_bytes(const tftq_plan *plan);
+const void *tftq_plan_table_host(const tftq_plan *plan);
+int tftq_plan_set_device_table(tftq_plan *plan, const void *device_table);
+
+/*
+ * fused_quantize_into_fp8 (quantization.py:531-588).  Reads the plan's
+ * tensors, writes every byte of packed[0 .. output_size): scales, codes, zero
+ * padding and zero padding rows, so `packed` needs no prior memset (the
+ * reference relies on torch.zeros, :567-571).  packed must be 4-byte aligned.
+ */
+int tftq_quantize(const tftq_plan *plan, void *packed, int64_t packed_bytes, void *stream);
+
+/*
+ * fused_reduce_fp8 (quantization.py:638-686).  packed holds ws slots, slot p =
+ * peer p's quantization of this rank's row slice.  Sums the slots in fp32 in
+ * the order rank, rank+1, ... (wrapping, :405-407), requantizes and overwrites
+ * slot `rank` (scale and codes of every row, padding rows included).  is_avg
+ * != 0 divides by ws (:682).  The plan's tensor pointers are not used.
+ */
+int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank,
+                int is_avg, void *stream);
+
+/*
+ * fused_dequantize_from_fp8 (quantization.py:591-635).  Writes
+ * cast(float(code) / scale) into the plan's tensors (all m_i real rows).
+ */
+int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
+                    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFTQ_H */

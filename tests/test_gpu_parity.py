@@ -1,0 +1,337 @@
+"""Parity of the HIP path (through torchft_amd.quantization -> ctypes ->
+libtftq.so) with the CPU checker, on a gfx950 GPU.
+
+Bar: every byte of the packed buffer after quantize and after reduce, and every
+element after dequantize, equals the checker's.  (The stated tolerance for
+reduce / dequantize is one fp8-e4m3 ULP of the row scale, 32 / s; the kernels
+reproduce the summation order and use an exact division, so the tests demand
+equality and report nothing looser.)
+"""
+
+import ctypes
+import json
+import os
+
+import pytest
+import torch
+from torch.distributed import ReduceOp
+
+import sim
+import workloads
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+NT = min(16, os.cpu_count() or 1)
+
+
+@pytest.fixture(scope="module")
+def q():
+    assert torch.cuda.is_available(), "GPU tests need a gfx950 device"
+    from torchft_amd import _lib, quantization
+    assert _lib.load().tftq_check_device() == 0, "device is not gfx950"
+    return quantization
+
+
+def dev(ts):
+    return [t.cuda() for t in ts]
+
+
+def same_bytes(a: torch.Tensor, b: torch.Tensor, what=""):
+    a = a.detach().cpu().contiguous().view(-1).view(torch.uint8)
+    b = b.detach().cpu().contiguous().view(-1).view(torch.uint8)
+    assert a.numel() == b.numel(), what
+    if not torch.equal(a, b):
+        bad = (a != b).nonzero().flatten()
+        raise AssertionError(f"{what}: {bad.numel()} bytes differ, first at {bad[:8].tolist()}: "
+                             f"got {a[bad[:8]].tolist()} want {b[bad[:8]].tolist()}")
+
+
+def full_check(q, oracle, peers_cpu, ws, op, ranks=None):
+    """Quantize every peer, reduce on `ranks`, dequantize; all against the checker."""
+    peers_gpu = [dev(t) for t in peers_cpu]
+    qs_g, red_g, gath_g = sim.allreduce(q, peers_gpu, ws, op, ranks)
+    qs_c, red_c, gath_c = sim.allreduce(oracle, [list(t) for t in peers_cpu], ws, op, ranks, nthreads=NT)
+    for p, (a, b) in enumerate(zip(qs_g, qs_c)):
+        same_bytes(a, b, f"quantize peer {p}")
+    for r in red_c:
+        same_bytes(red_g[r], red_c[r], f"reduce rank {r}")
+    if ranks is None:
+        outs_g = [torch.full_like(t, 7.0) for t in peers_gpu[0]]
+        outs_c = [torch.full_like(t, 7.0) for t in peers_cpu[0]]
+        q.fused_dequantize_from_fp8(outs_g, gath_g, ws)
+        oracle.fused_dequantize_from_fp8(outs_c, gath_c, ws, nthreads=NT)
+        for i, (a, b) in enumerate(zip(outs_g, outs_c)):
+            same_bytes(a, b, f"dequantize tensor {i}")
+        return outs_g
+    return None
+
+
+# ---- the fp8 convert instruction against the checker ------------------------
+def test_hw_fp8_convert_matches_checker(q, oracle):
+    """Rows whose amax is exactly 448 get scale 1.0, so the codes are the raw
+    hardware conversion of the inputs: all bf16 patterns up to 464 in magnitude,
+    a dense sweep around the overflow boundary, ties and subnormals."""
+    allbf = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).to(torch.float32)
+    allbf = allbf[allbf.abs() <= 448.0]
+    edge = torch.linspace(440.0, 448.0, 20001)
+    sub = torch.linspace(0, 2 ** -5, 40001)
+    g = torch.Generator().manual_seed(9)
+    rnd = (torch.rand(300000, generator=g) * 2 - 1) * 448.0
+    ties = torch.tensor([17.0, 19.0, 1.5 * 2 ** -9, 2.5 * 2 ** -9, 2 ** -10, 2 ** -10 * 1.0001,
+                         2 ** -6 * 0.9999, 0.0, -0.0, 1e-30, -1e-30, 1e-45])
+    x = torch.cat([allbf, edge, -edge, sub, -sub, rnd, ties])
+    n = 1023
+    rows = -(-x.numel() // n)
+    x = torch.cat([x, torch.zeros(rows * n - x.numel())]).view(rows, n)
+    x = torch.cat([x, torch.full((rows, 1), 448.0)], dim=1).contiguous()  # amax = 448 -> s = 1
+    got = q.fused_quantize_into_fp8([x.cuda()], 1)
+    want = oracle.fused_quantize_into_fp8([x], 1)
+    same_bytes(got, want, "hw convert")
+    assert (want.view(rows, -1)[:, :4].contiguous().view(torch.float32) == 1.0).all()
+
+
+# ---- golden vectors through the GPU ------------------------------------------
+def test_golden_vectors_gpu(q):
+    kat = json.load(open(os.path.join(HERE, "golden", "kat.json")))
+
+    def from_hex(h, dtype=torch.uint8):
+        return torch.frombuffer(bytearray(bytes.fromhex(h)), dtype=dtype).clone()
+
+    k = kat["kat1_quantize"]
+    x = from_hex(k["input_hex"]).view(torch.float32).view(1, 4).cuda()
+    assert bytes(q.fused_quantize_into_fp8([x], 1).cpu().tolist()).hex() == k["packed_hex"]
+    for name, op in (("sum", ReduceOp.SUM), ("avg", ReduceOp.AVG)):
+        k = kat[f"kat2_reduce_{name}"]
+        recv = from_hex(k["recv_hex"]).cuda()
+        q.fused_reduce_fp8([torch.empty(2, 4, device="cuda")], recv, 2, 0, op)
+        assert bytes(recv.cpu().tolist()).hex() == k["reduced_hex"]
+        out = torch.zeros(1, 4, device="cuda")
+        q.fused_dequantize_from_fp8([out], recv[:8].clone(), 1)
+        assert bytes(out.cpu().view(torch.uint8).flatten().tolist()).hex() == k["dequant_slot0_hex"]
+    for key in ("kat3_zero_row", "kat3_n1_rows"):
+        k = kat[key]
+        x = from_hex(k["input_hex"]).view(torch.float32).view(*k["shape"]).cuda()
+        assert bytes(q.fused_quantize_into_fp8([x], 1).cpu().tolist()).hex() == k["packed_hex"]
+    DT = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+    for dt in DT:
+        k = kat[f"odd_{dt}"]
+        ins = [from_hex(h).view(DT[dt]).view(*s).cuda() for h, s in zip(k["inputs_hex"], k["shapes"])]
+        buf = q.fused_quantize_into_fp8(list(ins), k["ws"])
+        assert bytes(buf.cpu().tolist()).hex() == k["packed_hex"]
+        red = buf.clone()
+        q.fused_reduce_fp8(list(ins), red, k["ws"], 2, ReduceOp.AVG)
+        assert bytes(red.cpu().tolist()).hex() == k["reduced_rank2_avg_hex"]
+        outs = [torch.zeros_like(t) for t in ins]
+        q.fused_dequantize_from_fp8(list(outs), buf, k["ws"])
+        for o, h in zip(outs, k["dequant_hex"]):
+            assert bytes(o.cpu().contiguous().view(torch.uint8).flatten().tolist()).hex() == h
+
+
+# ---- BASELINE configurations ---------------------------------------------------
+def test_cfg1_cpu_plumbing_shapes(q, oracle):
+    peers = [workloads.cfg1(s) for s in (0, 1)]
+    outs = full_check(q, oracle, peers, 2, ReduceOp.SUM)
+    ref = peers[0][0] + peers[1][0]
+    rowmax = ref.abs().amax(dim=1, keepdim=True)
+    assert ((outs[0].cpu() - ref).abs() / rowmax).max() < 0.13
+
+
+def test_cfg2_bf16_4096x4096_avg(q, oracle):
+    peers = [workloads.cfg2(s) for s in range(8)]
+    full_check(q, oracle, peers, 8, ReduceOp.AVG)
+
+
+@pytest.mark.parametrize("op", [ReduceOp.SUM, ReduceOp.AVG])
+def test_cfg3_llama_layer_eighth(q, oracle, op):
+    """All nine tensors at full row length, one eighth of the rows."""
+    peers = [workloads.cfg3(s, scale_rows=0.125) for s in range(8)]
+    full_check(q, oracle, peers, 8, op)
+
+
+def test_cfg4_diloco_two_layers(q, oracle):
+    peers = [workloads.cfg4(s, layers=2, vocab=4000) for s in range(4)]
+    assert len(peers[0]) == 21  # more than 16 tensors: descriptor table in device memory
+    full_check(q, oracle, peers, 4, ReduceOp.AVG)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_cfg5_edge_case_stress(q, oracle, dtype):
+    shapes = workloads.cfg5_shapes(600)
+    peers = [workloads.cfg5(s, dtype, shapes) for s in range(16)]
+    full_check(q, oracle, peers, 16, ReduceOp.SUM, ranks=[0, 7, 15])
+    full_check(q, oracle, peers[:2] * 8, 16, ReduceOp.SUM)
+
+
+# ---- the reference's own test matrix (quantization_test.py:107-131) ---------------
+def _views(size):
+    return [(m, size // m) for m in range(1 if size % 2 == 0 else 2, size) if size % m == 0]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("op", [ReduceOp.AVG, ReduceOp.SUM])
+@pytest.mark.parametrize("tensor_size,multiplier", [(128, 1.0), (512, 100.0), (4096, 1000.0)])
+def test_reference_matrix(q, oracle, dtype, op, tensor_size, multiplier):
+    """Shapes and inputs of QuantizationTest.run_test: uniform [0, multiplier),
+    three tensors, every 2-D factorisation; world size 2 with identical peers.
+    Checked bit for bit against the checker and with the reference's own
+    criterion (mean relative error <= 0.05, :96-105)."""
+    g = torch.Generator().manual_seed(tensor_size)
+    inp = (torch.rand(3 * tensor_size, generator=g) * multiplier).to(dtype)
+    views = _views(tensor_size)
+    # every view appears in some combination (the full cross product has len(views)^3 entries)
+    combos = [(views[i], views[(i * 7 + 3) % len(views)], views[-1 - i]) for i in range(len(views))]
+    for split in combos:
+        ins = [t.view(*s).clone() for s, t in zip(split, torch.split(inp, tensor_size))]
+        outs = full_check(q, oracle, [ins, ins], 2, op)
+        out = torch.cat([o.reshape(-1) for o in outs]).cpu().float()
+        ref = inp.float() * (2 if op == ReduceOp.SUM else 1)
+        assert not torch.isnan(out).any()
+        assert ((ref - out).abs() / (ref + 1e-7)).mean() <= 0.05
+
+
+# ---- layouts the fast paths do not take ----------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_strided_and_misaligned_inputs(q, oracle, dtype):
+    g = torch.Generator().manual_seed(11)
+    base = (torch.randn(300, 700, generator=g)).to(dtype)
+    flat = (torch.randn(5000, generator=g)).to(dtype)
+    cpu_views = [base[::2, 1:600:3], base.t()[3:170], base[5:6, :], flat[1:4097].view(64, 64), flat[3:3 + 77]]
+    gbase, gflat = base.cuda(), flat.cuda()
+    gpu_views = [gbase[::2, 1:600:3], gbase.t()[3:170], gbase[5:6, :], gflat[1:4097].view(64, 64), gflat[3:3 + 77]]
+    a = q.fused_quantize_into_fp8(list(gpu_views), 4)
+    b = oracle.fused_quantize_into_fp8(list(cpu_views), 4)
+    same_bytes(a, b, "strided quantize")
+    # dequantize into strided, non-overlapping destinations
+    ob, of = torch.zeros(300, 700, dtype=dtype), torch.zeros(5000, dtype=dtype)
+    gob, gof = ob.cuda(), of.cuda()
+    cpu_out = [ob[::2, 1:600:3], of[1:4097].view(64, 64)]
+    gpu_out = [gob[::2, 1:600:3], gof[1:4097].view(64, 64)]
+    src_c = [cpu_views[0], cpu_views[3]]
+    buf = oracle.fused_quantize_into_fp8(list(src_c), 4)
+    oracle.fused_dequantize_from_fp8(list(cpu_out), buf, 4)
+    q.fused_dequantize_from_fp8(list(gpu_out), buf.cuda(), 4)
+    same_bytes(gob, ob, "strided dequantize base")
+    same_bytes(gof, of, "strided dequantize flat")
+
+
+@pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (3, ReduceOp.AVG), (5, ReduceOp.SUM),
+                                   (6, ReduceOp.AVG), (70, ReduceOp.AVG), (64, ReduceOp.SUM)])
+def test_group_sizes(q, oracle, ws, op):
+    g = torch.Generator().manual_seed(ws)
+    shapes = [(37, 256), (5, 4096), (130,), (3, 14336), (9, 33), (2, 1024)]
+    peers = [[(torch.randn(s, generator=g) * (1 + p % 5)).to(torch.bfloat16) for s in shapes]
+             for p in range(ws)]
+    ranks = None if ws <= 6 else [0, ws // 2, ws - 1]
+    full_check(q, oracle, peers, ws, op, ranks)
+
+
+def test_long_rows(q, oracle):
+    """Rows longer than the register-resident paths hold: 20000 and 70000 columns."""
+    g = torch.Generator().manual_seed(21)
+    for dtype in (torch.bfloat16, torch.float32):
+        peers = [[(torch.randn(5, 20000, generator=g)).to(dtype),
+                  (torch.randn(3, 70000, generator=g)).to(dtype)] for _ in range(2)]
+        full_check(q, oracle, peers, 2, ReduceOp.AVG)
+
+
+def test_extreme_scales_and_denormals(q, oracle):
+    """Row maxima far outside the range where the fast division applies
+    (scale exponent beyond +-64), fp32 denormal inputs, all-zero rows."""
+    g = torch.Generator().manual_seed(31)
+    mags = torch.tensor([1e-38, 1e-33, 1e-30, 1e-25, 1e-20, 1.0, 1e18, 1e22, 1e25, 1e30, 3e38])
+    x = torch.randn(len(mags), 4096, generator=g).clamp(-3, 3) / 3 * mags[:, None]
+    x = torch.cat([x, torch.zeros(1, 4096), torch.full((1, 4096), 1e-45)])
+    y = torch.randn(len(mags) + 2, 33, generator=g).clamp(-3, 3) / 3 * torch.cat([mags, mags[:2]])[:, None]
+    z = (torch.randn(len(mags) + 2, generator=g).clamp(-3, 3) / 3) * torch.cat([mags, mags[:2]])
+    peers = [[x * (p + 1) / 4, y * (p + 1) / 4, z * (p + 1) / 4] for p in range(4)]
+    full_check(q, oracle, peers, 4, ReduceOp.SUM)
+    full_check(q, oracle, peers, 4, ReduceOp.AVG)
+    full_check(q, oracle, peers[:1], 1, ReduceOp.SUM)
+
+
+def test_empty_and_ragged(q, oracle):
+    peers = [[torch.zeros(0, 5), torch.ones(3, 0), torch.arange(7.0), torch.ones(1, 1)] for _ in range(2)]
+    full_check(q, oracle, peers, 2, ReduceOp.SUM)
+    full_check(q, oracle, peers * 2, 4, ReduceOp.AVG)
+
+
+# ---- properties at full size ---------------------------------------------------
+def test_cfg3_full_size(q, oracle):
+    """The whole Llama-3-8B layer bucket (218 M elements, ws = 8): peer 0's packed
+    buffer and one rank's reduction against the checker, then size-independent
+    properties of the full round trip on the GPU."""
+    ws = 8
+    peers_gpu = []
+    q0_cpu = None
+    for s in range(ws):
+        t = workloads.cfg3(s)
+        if s == 0:
+            q0_cpu = oracle.fused_quantize_into_fp8(list(t), ws, nthreads=NT)
+            peer0_cpu = t
+        peers_gpu.append(dev(t))
+    qs = sim.quantize_peers(q, peers_gpu, ws)
+    assert qs[0].numel() == 218341376
+    same_bytes(qs[0], q0_cpu, "cfg3 quantize peer 0")
+    del q0_cpu
+    rank = 5
+    recv = sim.recv_buffer(qs, rank, ws)
+    recv_cpu = recv.cpu()
+    q.fused_reduce_fp8(list(peers_gpu[0]), recv, ws, rank, ReduceOp.AVG)
+    oracle.fused_reduce_fp8(list(peer0_cpu), recv_cpu, ws, rank, ReduceOp.AVG, nthreads=NT)
+    same_bytes(recv, recv_cpu, "cfg3 reduce rank 5")
+    # round trip of peer 0 alone: quantize -> dequantize is within half an fp8 ULP per row
+    outs = [torch.empty_like(t) for t in peers_gpu[0]]
+    q.fused_dequantize_from_fp8(outs, qs[0], ws)
+    for x, o in zip(peers_gpu[0], outs):
+        xf, of = x.float().view(x.shape[0], -1), o.float().view(x.shape[0], -1)
+        amax = xf.abs().amax(dim=1, keepdim=True)
+        # fp8 half-ULP (2^-4 relative, 2^-10/s absolute) plus the bf16 store rounding (2^-9)
+        tol = torch.maximum(xf.abs() * (2 ** -4 + 2 ** -8), amax * (2 ** -10 / 448.0) * 1.01)
+        assert ((xf - of).abs() <= tol).all()
+    # idempotence: quantizing the dequantized tensors reproduces the codes (scales may move an ulp)
+    q2 = q.fused_quantize_into_fp8(list(outs), ws)
+    d2 = [torch.empty_like(t) for t in outs]
+    q.fused_dequantize_from_fp8(d2, q2, ws)
+    for a, b in zip(outs, d2):
+        assert torch.equal(a, b)
+
+
+# ---- memory safety around the packed buffer ---------------------------------------
+def test_no_write_outside_packed_buffer(q):
+    """Calls the C ABI with a packed buffer placed between two canary zones."""
+    from torchft_amd import _lib
+    L = _lib.load()
+    g = torch.Generator().manual_seed(41)
+    shapes = [(37, 4096), (5, 333), (19,), (64, 64), (3, 14336)]
+    ts = [torch.randn(s, generator=g).to(torch.bfloat16).cuda() for s in shapes]
+    ts = [t if t.dim() == 2 else t.unsqueeze(1) for t in ts]
+    ws, T, guard = 4, len(ts), 4096
+    ptrs = (ctypes.c_void_p * T)(*[t.data_ptr() for t in ts])
+    sh = (ctypes.c_int64 * (2 * T))(*[v for t in ts for v in t.shape])
+    st = (ctypes.c_int64 * (2 * T))(*[v for t in ts for v in t.stride()])
+    h = ctypes.c_void_p()
+    assert L.tftq_plan_create(2, T, ptrs, sh, st, ws, ctypes.byref(h)) == 0
+    size = L.tftq_plan_output_size(h)
+    arena = torch.full((size + 2 * guard,), 0xA5, dtype=torch.uint8, device="cuda")
+    packed = arena[guard:guard + size]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert L.tftq_quantize(h, ctypes.c_void_p(packed.data_ptr()), size, stream) == 0
+    assert L.tftq_reduce(h, ctypes.c_void_p(packed.data_ptr()), size, 1, 1, stream) == 0
+    assert L.tftq_dequantize(h, ctypes.c_void_p(packed.data_ptr()), size, stream) == 0
+    torch.cuda.synchronize()
+    assert (arena[:guard] == 0xA5).all() and (arena[guard + size:] == 0xA5).all()
+    assert L.tftq_quantize(h, ctypes.c_void_p(packed.data_ptr()), size - 4, stream) == -4
+    assert L.tftq_reduce(h, ctypes.c_void_p(packed.data_ptr()), size, 4, 0, stream) == -1
+    L.tftq_plan_destroy(h)
+
+
+def test_wrapper_errors_on_gpu(q):
+    x = [torch.zeros(8, 8, device="cuda")]
+    buf = q.fused_quantize_into_fp8(x, 2)
+    with pytest.raises(AssertionError, match="Output size does not match"):
+        q.fused_reduce_fp8(x, buf[:-4], 2, 0)
+    with pytest.raises(AssertionError, match="Output size does not match"):
+        q.fused_dequantize_from_fp8(x, buf[:-4], 2)
+    with pytest.raises(RuntimeError):
+        q.fused_reduce_fp8(x, buf, 2, 2)

@@ -1,0 +1,85 @@
+// Shared between the host-side planner (tftq_plan.cpp) and the HIP kernels
+// (tftq_kernels.hip).  Not part of the public ABI.
+#pragma once
+
+#include <stdint.h>
+
+#include <vector>
+
+// Stages of the path, used to index per-stage fields of a segment.
+enum : int { ST_Q = 0, ST_R = 1, ST_D = 2 };
+
+// How the rows of one tensor are mapped onto lanes.  "Team" = the lanes that
+// cooperate on one row.  VEC kinds need contiguous 16-byte aligned rows whose
+// length is a whole number of 16-byte vectors; GEN kinds take any strides.
+enum : uint8_t {
+    K_NONE = 0,
+    K_VEC8 = 1,    // 8 lanes per row, 32 rows per workgroup
+    K_VEC64 = 2,   // one wavefront per row, 4 rows per workgroup
+    K_VEC256 = 3,  // one workgroup per row (also loops over rows too long for registers)
+    K_GEN1 = 4,    // one lane per row, 256 rows per workgroup
+    K_GEN8 = 5,    // 8 lanes per row
+    K_GEN64 = 6,   // one wavefront per row
+    K_GEN256 = 7,  // one workgroup per row (reduce only)
+};
+
+static inline int tftq_team_of(uint8_t kind)
+{
+    switch (kind) {
+    case K_VEC8: case K_GEN8: return 8;
+    case K_VEC64: case K_GEN64: return 64;
+    case K_VEC256: case K_GEN256: return 256;
+    case K_GEN1: return 1;
+    default: return 256;
+    }
+}
+
+constexpr int TFTQ_WG = 256;       // threads per workgroup, all kernels
+constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
+
+// One tensor of the list.  64 bytes.
+struct Seg {
+    uint64_t ptr;        // device address of element (0,0); 0 for reduce-only plans
+    int64_t slot_off;    // byte offset of this tensor's rows inside every slot
+    int64_t row_stride;  // elements
+    int64_t col_stride;  // elements
+    int32_t m;           // real rows
+    int32_t n;           // columns
+    int32_t slice_rows;  // rows per slot = ceil(m / ws)
+    int32_t row_bytes;   // 4 + round_up(n, 4)
+    int32_t wg_begin[3]; // first workgroup of this segment, per stage
+    uint8_t kind[3];     // lane mapping, per stage
+    uint8_t pad;
+};
+static_assert(sizeof(Seg) == 64, "Seg must be 64 bytes");
+
+struct InlineTable {
+    Seg s[TFTQ_N_INLINE];
+};
+
+struct tftq_plan {
+    int dtype;
+    int esz;
+    int ws;
+    int nseg;
+    int64_t slot_size;
+    int64_t output_size;
+    int64_t max_rows;
+    int32_t nwg[3];
+    std::vector<Seg> segs;
+    const void *device_table;  // set by the caller when nseg > TFTQ_N_INLINE
+};
+
+// Kernel parameters common to the three stages.
+struct KParams {
+    const Seg *table;   // device table, or nullptr when the inline table is used
+    uint8_t *packed;
+    int64_t slot_size;
+    int32_t nseg;
+    int32_t nwg;
+    int32_t ws;
+    int32_t rank;
+    int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG general
+    float div;          // reduce: 1.0 or float(ws)
+    float inv_div;      // reduce: exact reciprocal when div_mode == 1
+};

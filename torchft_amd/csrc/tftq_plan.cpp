@@ -1,0 +1,164 @@
+// Host-side planner: layout arithmetic of the packed buffer and the partition
+// of rows into workgroups.  No HIP calls; compiles with any C++17 compiler.
+//
+// The layout restates _prepare_quantize_fp8 (torchft/quantization.py:486-503)
+// and the row addressing of the kernels (:108-123).  Offsets are 64-bit here;
+// the reference keeps them in int32 (:514-515).
+
+#include <limits.h>
+#include <string.h>
+
+#include <new>
+
+#include "../../include/tftq.h"
+#include "tftq_internal.h"
+
+static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+extern "C" int tftq_version(void) { return TFTQ_VERSION; }
+
+extern "C" const char *tftq_strerror(int code)
+{
+    switch (code) {
+    case 0: return "success";
+    case TFTQ_E_ARG: return "invalid argument";
+    case TFTQ_E_DTYPE: return "Only fp32, fp16 and bf16 are supported";
+    case TFTQ_E_SHAPE: return "tensor dimension out of range";
+    case TFTQ_E_SIZE: return "Output size does not match";
+    case TFTQ_E_NOMEM: return "out of host memory";
+    case TFTQ_E_NOTABLE: return "plan needs a device descriptor table";
+    case TFTQ_E_ARCH: return "device is not gfx950";
+    default: return code > 0 ? "HIP error" : "unknown error";
+    }
+}
+
+extern "C" int tftq_layout(int n_tensors, const int64_t *shapes, int ws, int64_t *slot_off,
+                           int64_t *slot_size, int64_t *output_size)
+{
+    if (n_tensors <= 0 || !shapes || ws <= 0) return TFTQ_E_ARG;
+    int64_t per_rank = 0;
+    for (int i = 0; i < n_tensors; i++) {
+        const int64_t m = shapes[2 * i], n = shapes[2 * i + 1];
+        if (m < 0 || n < 0 || m > INT32_MAX - ws || n > INT32_MAX - 8) return TFTQ_E_SHAPE;
+        const int64_t row_bytes = (cdiv64(n, 4) + 1) * 4;
+        if (slot_off) slot_off[i] = per_rank;
+        per_rank += cdiv64(m, ws) * row_bytes;
+        if (per_rank > (INT64_MAX / 2) / ws) return TFTQ_E_SHAPE;
+    }
+    if (slot_size) *slot_size = per_rank;
+    if (output_size) *output_size = per_rank * ws;
+    return 0;
+}
+
+static uint8_t pick_io_kind(const Seg &s, int esz)
+{
+    const int epv = 16 / esz;
+    const int64_t in_bytes = (int64_t)s.n * esz;
+    const bool vec_ok = s.ptr != 0 && s.n > 0 && s.n % epv == 0 && s.col_stride == 1 &&
+                        s.ptr % 16 == 0 && (s.m <= 1 || (s.row_stride * esz) % 16 == 0) &&
+                        in_bytes >= 64;
+    if (vec_ok) {
+        if (in_bytes <= 1024) return K_VEC8;
+        if (in_bytes <= 8192) return K_VEC64;
+        if (in_bytes <= 32768) return K_VEC256;
+    }
+    if (s.n <= 16) return K_GEN1;
+    if (s.n <= 128) return K_GEN8;
+    return K_GEN64;
+}
+
+static uint8_t pick_reduce_kind(const Seg &s)
+{
+    // one 16-byte vector of codes per lane and peer, except for the longest rows
+    const int ndw = s.row_bytes / 4 - 1;
+    if (ndw <= 4) return K_GEN1;
+    if (ndw <= 32) return K_GEN8;
+    if (ndw <= 256) return K_GEN64;
+    return K_GEN256;
+}
+
+extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
+                                const int64_t *shapes, const int64_t *strides, int ws,
+                                tftq_plan **out)
+{
+    if (!out) return TFTQ_E_ARG;
+    *out = nullptr;
+    if (dtype != TFTQ_F32 && dtype != TFTQ_F16 && dtype != TFTQ_BF16) return TFTQ_E_DTYPE;
+    if (n_tensors <= 0 || !shapes || !strides || ws <= 0) return TFTQ_E_ARG;
+
+    tftq_plan *p = new (std::nothrow) tftq_plan();
+    if (!p) return TFTQ_E_NOMEM;
+    p->dtype = dtype;
+    p->esz = dtype == TFTQ_F32 ? 4 : 2;
+    p->ws = ws;
+    p->nseg = n_tensors;
+    p->device_table = nullptr;
+    p->max_rows = 0;
+    try {
+        p->segs.resize((size_t)n_tensors);
+    } catch (...) {
+        delete p;
+        return TFTQ_E_NOMEM;
+    }
+    std::vector<int64_t> offs((size_t)n_tensors);
+    int rc = tftq_layout(n_tensors, shapes, ws, offs.data(), &p->slot_size, &p->output_size);
+    if (rc) {
+        delete p;
+        return rc;
+    }
+    int64_t wg[3] = {0, 0, 0};
+    for (int i = 0; i < n_tensors; i++) {
+        Seg &s = p->segs[(size_t)i];
+        memset(&s, 0, sizeof(s));
+        s.ptr = ptrs ? (uint64_t)(uintptr_t)ptrs[i] : 0;
+        s.slot_off = offs[(size_t)i];
+        s.m = (int32_t)shapes[2 * i];
+        s.n = (int32_t)shapes[2 * i + 1];
+        s.row_stride = strides[2 * i];
+        s.col_stride = strides[2 * i + 1];
+        s.slice_rows = (int32_t)cdiv64(s.m, ws);
+        s.row_bytes = (int32_t)((cdiv64(s.n, 4) + 1) * 4);
+        const int64_t m_pad = (int64_t)s.slice_rows * ws;
+        if (m_pad > p->max_rows) p->max_rows = m_pad;
+
+        s.kind[ST_Q] = s.kind[ST_D] = pick_io_kind(s, p->esz);
+        s.kind[ST_R] = pick_reduce_kind(s);
+        const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
+        for (int st = 0; st < 3; st++) {
+            s.wg_begin[st] = (int32_t)wg[st];
+            const int rows_per_wg = TFTQ_WG / tftq_team_of(s.kind[st]);
+            wg[st] += cdiv64(rows[st], rows_per_wg);
+            if (wg[st] > INT32_MAX - 16) {
+                delete p;
+                return TFTQ_E_SHAPE;
+            }
+        }
+    }
+    for (int st = 0; st < 3; st++) p->nwg[st] = (int32_t)wg[st];
+    *out = p;
+    return 0;
+}
+
+extern "C" void tftq_plan_destroy(tftq_plan *plan) { delete plan; }
+
+extern "C" int64_t tftq_plan_output_size(const tftq_plan *plan) { return plan ? plan->output_size : -1; }
+extern "C" int64_t tftq_plan_slot_size(const tftq_plan *plan) { return plan ? plan->slot_size : -1; }
+extern "C" int64_t tftq_plan_max_rows(const tftq_plan *plan) { return plan ? plan->max_rows : -1; }
+
+extern "C" int64_t tftq_plan_table_bytes(const tftq_plan *plan)
+{
+    if (!plan) return -1;
+    return plan->nseg > TFTQ_N_INLINE ? (int64_t)plan->nseg * (int64_t)sizeof(Seg) : 0;
+}
+
+extern "C" const void *tftq_plan_table_host(const tftq_plan *plan)
+{
+    return plan ? (const void *)plan->segs.data() : nullptr;
+}
+
+extern "C" int tftq_plan_set_device_table(tftq_plan *plan, const void *device_table)
+{
+    if (!plan) return TFTQ_E_ARG;
+    plan->device_table = device_table;
+    return 0;
+}

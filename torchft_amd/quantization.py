@@ -1,0 +1,205 @@
+"""FP8 quantized-collective kernels: host side.
+
+Drop-in for ``torchft/quantization.py``: the same three public functions with
+the same positional signatures, the same packed-buffer layout and the same
+assertion messages (quantization.py:463-489, 621, 672), backed by hand-written
+gfx950 kernels in ``libtftq.so`` instead of Triton.  Differences a caller can
+observe:
+
+* only the fp8-e4m3fn / 448 branch exists (quantization.py:30-41; gfx950 reports
+  capability (9, 5)); the int8 / 127 branch for older GPUs is not built;
+* the packed buffer is allocated uninitialised and every byte of it is written
+  by the quantize kernel, instead of ``torch.zeros`` plus a kernel
+  (quantization.py:567-571); the bytes are identical;
+* the per-call host work of ``_prepare_quantize_fp8`` (four device tables and
+  five allocations per call, quantization.py:505-517) is replaced by a cached
+  plan; lists of up to 16 tensors need no device metadata at all.
+
+There is no CPU or eager fallback: without the HIP library and a gfx950 device
+the functions raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from collections import OrderedDict
+
+import torch
+from torch.distributed import ReduceOp
+
+from . import _lib
+
+SCALE_DTYPE: torch.dtype = torch.float32
+SCALE_DTYPE_BYTES: int = 4
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+_PLAN_CACHE_SIZE = 64
+
+
+class _Plan:
+    """Owns a ``tftq_plan`` and, for long tensor lists, its device table."""
+
+    __slots__ = ("handle", "output_size", "slot_size", "max_rows", "table", "_lib")
+
+    def __init__(self, lib, handle, table):
+        self._lib = lib
+        self.handle = handle
+        self.table = table
+        self.output_size = lib.tftq_plan_output_size(handle)
+        self.slot_size = lib.tftq_plan_slot_size(handle)
+        self.max_rows = lib.tftq_plan_max_rows(handle)
+
+    def __del__(self):
+        try:
+            if self.handle:
+                self._lib.tftq_plan_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+_cache_lock = threading.Lock()
+_plan_cache: "OrderedDict[tuple, _Plan]" = OrderedDict()
+
+
+def _check(rc: int, what: str) -> None:
+    if rc == 0:
+        return
+    if rc == -4:  # TFTQ_E_SIZE
+        raise AssertionError("Output size does not match")
+    raise RuntimeError(f"{what} failed: {_lib.strerror(rc)}")
+
+
+def _validate(inputs: list[torch.Tensor]) -> tuple[torch.device, torch.dtype]:
+    # quantization.py:462-478, same order and messages
+    i_num = len(inputs)
+    assert i_num > 0, "At least one input tensor is required"
+    device = inputs[0].device
+    dtype = inputs[0].dtype
+    for i in range(1, i_num):
+        assert inputs[i].device == inputs[i - 1].device, "All inputs must be on the same device"
+        assert inputs[i].dtype == inputs[i - 1].dtype, "All inputs must be on the same dtype"
+    assert dtype in _DTYPE_CODE, "Only fp32, fp16 and bf16 are supported"
+    for i in range(i_num):
+        # 1-D tensors become [k, 1] in the caller's list (quantization.py:487-488)
+        if inputs[i].dim() == 1:
+            inputs[i] = inputs[i].unsqueeze(1)
+        assert inputs[i].dim() == 2, "Only 2D tensors are supported"
+    return device, dtype
+
+
+def _prepare(inputs: list[torch.Tensor], all_reduce_group_size: int) -> tuple[_Plan, torch.device]:
+    """Counterpart of ``_prepare_quantize_fp8`` (quantization.py:431-528)."""
+    device, dtype = _validate(inputs)
+    if device.type != "cuda":
+        raise RuntimeError(
+            "torchft_amd.quantization needs tensors on a gfx950 GPU; there is no CPU path")
+    ws = int(all_reduce_group_size)
+    key = (device.index, dtype, ws,
+           tuple((t.data_ptr(), t.shape[0], t.shape[1], t.stride(0), t.stride(1)) for t in inputs))
+    with _cache_lock:
+        plan = _plan_cache.get(key)
+        if plan is not None:
+            _plan_cache.move_to_end(key)
+            return plan, device
+
+    lib = _lib.load()
+    T = len(inputs)
+    ptrs = (ctypes.c_void_p * T)()
+    shapes = (ctypes.c_int64 * (2 * T))()
+    strides = (ctypes.c_int64 * (2 * T))()
+    for i, t in enumerate(inputs):
+        ptrs[i] = t.data_ptr()
+        shapes[2 * i], shapes[2 * i + 1] = t.shape
+        strides[2 * i], strides[2 * i + 1] = t.stride()
+    handle = ctypes.c_void_p()
+    _check(lib.tftq_plan_create(_DTYPE_CODE[dtype], T, ptrs, shapes, strides, ws,
+                                ctypes.byref(handle)), "tftq_plan_create")
+    table = None
+    nbytes = lib.tftq_plan_table_bytes(handle)
+    if nbytes > 0:
+        host = (ctypes.c_uint8 * nbytes).from_address(lib.tftq_plan_table_host(handle))
+        # synchronous copy: the plan may be used from any stream afterwards
+        table = torch.frombuffer(host, dtype=torch.uint8).to(device)
+        _check(lib.tftq_plan_set_device_table(handle, ctypes.c_void_p(table.data_ptr())),
+               "tftq_plan_set_device_table")
+    plan = _Plan(lib, handle, table)
+    with _cache_lock:
+        _plan_cache[key] = plan
+        while len(_plan_cache) > _PLAN_CACHE_SIZE:
+            _plan_cache.popitem(last=False)
+    return plan, device
+
+
+def _stream_ptr(device: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _check_packed(output: torch.Tensor, plan: _Plan) -> None:
+    assert output.shape[0] == plan.output_size, "Output size does not match"
+    if output.dtype != torch.uint8 or not output.is_contiguous():
+        raise RuntimeError("the packed buffer must be a contiguous uint8 tensor")
+
+
+def fused_quantize_into_fp8(
+    inputs: list[torch.Tensor], all_reduce_group_size: int
+) -> torch.Tensor:
+    """
+    Quantizes every row of every input tensor to fp8-e4m3fn with its own fp32
+    scale and packs ``[scale][codes][pad]`` rows into one uint8 tensor laid out
+    as ``all_reduce_group_size`` equal slots (quantization.py:531-588).
+
+    Args:
+        inputs: tensors to quantize (1-D or 2-D, one dtype, one device)
+        all_reduce_group_size: size of the all-reduce group
+
+    Returns:
+        the packed uint8 tensor (``numel() % all_reduce_group_size == 0``)
+    """
+    plan, device = _prepare(inputs, all_reduce_group_size)
+    with torch.cuda.device(device):
+        # float32 storage like the reference (:567-571) so that scales are aligned
+        output = torch.empty(plan.output_size // SCALE_DTYPE_BYTES, device=device,
+                             dtype=SCALE_DTYPE).view(torch.uint8)
+        _check(plan._lib.tftq_quantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                       plan.output_size, _stream_ptr(device)), "tftq_quantize")
+    return output
+
+
+def fused_dequantize_from_fp8(
+    inputs: list[torch.Tensor], output: torch.Tensor, all_reduce_group_size: int
+) -> None:
+    """
+    Dequantizes the packed tensor ``output`` into ``inputs`` in place
+    (quantization.py:591-635).  The tensors must have the shapes that were
+    quantized.
+    """
+    plan, device = _prepare(inputs, all_reduce_group_size)
+    _check_packed(output, plan)
+    with torch.cuda.device(device):
+        _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                         plan.output_size, _stream_ptr(device)),
+               "tftq_dequantize")
+
+
+def fused_reduce_fp8(
+    inputs: list[torch.Tensor],
+    output: torch.Tensor,
+    all_reduce_group_size: int,
+    all_reduce_rank: int,
+    reduce_op: ReduceOp = ReduceOp.SUM,
+) -> None:
+    """
+    Sums the ``all_reduce_group_size`` slots of ``output`` in fp32, requantizes
+    and stores the result in slot ``all_reduce_rank`` (quantization.py:638-686).
+    Any ``reduce_op`` other than SUM averages (quantization.py:682).
+    ``inputs`` only supplies the shapes.
+    """
+    plan, device = _prepare(inputs, all_reduce_group_size)
+    _check_packed(output, plan)
+    is_avg = 0 if reduce_op == ReduceOp.SUM else 1
+    with torch.cuda.device(device):
+        _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                     plan.output_size, int(all_reduce_rank), is_avg,
+                                     _stream_ptr(device)), "tftq_reduce")
