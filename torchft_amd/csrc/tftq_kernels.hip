@@ -134,6 +134,14 @@ DEV DivCoef make_div(float s)
 
 DEV float div_fast(float f, float r, float r_lo) { return __builtin_fmaf(f, r, f * r_lo); }
 
+// Same, with the sign of a zero numerator kept (-0 / s = -0 for s > 0; the fma
+// form gives +0).  The sum in reduce cannot tell the two zeros apart, the
+// stored result of dequantize can.
+DEV float div_fast_signed(float f, float r, float r_lo)
+{
+    return __builtin_copysignf(div_fast(f, r, r_lo), f);
+}
+
 // four e4m3 codes -> four floats
 DEV void unpack_fp8x4(u32 w, float (&f)[4])
 {
@@ -216,11 +224,19 @@ template <> struct Elem<f16_tag> {
         unpack2(v.x, f[0], f[1]); unpack2(v.y, f[2], f[3]);
         unpack2(v.z, f[4], f[5]); unpack2(v.w, f[6], f[7]);
     }
+    // The value is first rounded to binary32, then to binary16.  Hide the
+    // producer from the compiler: it would otherwise fuse fma + convert into
+    // v_fma_mixlo_f16, which rounds once and differs in the last bit.
+    DEV static float opaque(float x)
+    {
+        asm("" : "+v"(x));
+        return x;
+    }
     DEV static u32 pack2(float a, float b)
     {
         f16x2 h;
-        h.x = (_Float16)a;  // round to nearest even
-        h.y = (_Float16)b;
+        h.x = (_Float16)opaque(a);  // round to nearest even
+        h.y = (_Float16)opaque(b);
         return __builtin_bit_cast(u32, h);
     }
     DEV static u32x4 pack(const float (&f)[8])
@@ -234,7 +250,7 @@ template <> struct Elem<f16_tag> {
     }
     DEV static void store(uint64_t base, int64_t idx, float v)
     {
-        as_global<_Float16>(base)[idx] = (_Float16)v;
+        as_global<_Float16>(base)[idx] = (_Float16)opaque(v);
     }
 };
 
@@ -414,7 +430,7 @@ DEV u32x4 dequant_vec_unit(GLOBAL const u32 *payload, int idx, float r, float r_
         float f[4];
         unpack_fp8x4(payload[idx], f);
 #pragma unroll
-        for (int e = 0; e < 4; e++) o[e] = div_fast(f[e], r, r_lo);
+        for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], r, r_lo);
     } else {
         const u32x2 w = *(GLOBAL const u32x2_a4 *)(payload + 2 * idx);
         float f[4], g[4];
@@ -422,8 +438,8 @@ DEV u32x4 dequant_vec_unit(GLOBAL const u32 *payload, int idx, float r, float r_
         unpack_fp8x4(w.y, g);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            o[e] = div_fast(f[e], r, r_lo);
-            o[4 + e] = div_fast(g[e], r, r_lo);
+            o[e] = div_fast_signed(f[e], r, r_lo);
+            o[4 + e] = div_fast_signed(g[e], r, r_lo);
         }
     }
     return Elem<T>::pack(o);
@@ -442,7 +458,7 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
     if (c.fast) {
         for (int col = lane; col < s.n; col += TEAM) {
             const float f = __builtin_amdgcn_cvt_f32_fp8((int)in[4 + col], 0);
-            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, div_fast(f, c.r, c.r_lo));
+            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, div_fast_signed(f, c.r, c.r_lo));
         }
     } else {
 #pragma nounroll
