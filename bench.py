@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 quantized-collective hot path on one MI355X.
+
+One step = one pass of the path over one gradient bucket, as one rank of an
+8-way quantized all-reduce sees it (torchft/collectives.py:364-412):
+    quantize   the rank's tensors          -> packed buffer A
+    reduce     the received buffer B (8 peer slots) in place, own slot rewritten
+    dequantize the gathered buffer G       -> the rank's tensors
+The two collectives are not part of the step: B and G are prepared beforehand on
+the same GPU from 8 independently seeded peers.  Inputs are resident in HBM
+before the timed region.  The step rotates over several buffer sets so that the
+256 MB last-level cache cannot hold the working set of the next step ("cold").
+
+Workload: BASELINE configuration 3, the Llama-3-8B decoder-layer gradient
+bucket (9 bf16 tensors, 218 112 000 elements, per-row std log-uniform in
+[1e-5, 1e-1]), world size 8, reduce op AVG.
+
+Prints one JSON line.  `value` is algorithmic bytes of the three stages divided
+by the wall time of a step; `roofline` is the quantize kernel against the 8 TB/s
+HBM peak; `stages` has the same figure for each kernel; `cpu_baseline` is the
+CPU checker (oracle/, a port of the reference arithmetic - the reference has no
+CPU implementation) on the host cores, on a bounded sample of the same bucket.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--sets", type=int, default=3, help="buffer sets the steps rotate over")
+    ap.add_argument("--rank", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=float, default=1.0,
+                    help="fraction of the bucket's rows the CPU baseline runs on")
+    return ap.parse_args()
+
+
+def cpu_baseline(fraction: float):
+    """Times the CPU checker on `fraction` of the rows of every tensor of the bucket."""
+    import torch
+    from torch.distributed import ReduceOp
+
+    import workloads
+    from oracle import oracle
+
+    ws = 8
+    nthreads = max(1, min(oracle.max_threads(), os.cpu_count() or 1))
+    tensors = workloads.cfg3(0, scale_rows=fraction)
+    ab = workloads.algorithmic_bytes(tensors, ws)
+    outs = [torch.empty_like(t) for t in tensors]
+    qbuf = oracle.fused_quantize_into_fp8(list(tensors), ws, nthreads=nthreads)  # warm-up, page-in
+    recv = qbuf.clone()  # a full buffer of 8 slots stands in for the received one
+    oracle.fused_dequantize_from_fp8(outs, qbuf, ws, nthreads=nthreads)
+    tq = tr = td = 0.0
+    passes = 0
+    while passes < 2 or (tq + tr + td < 10.0 and passes < 400):
+        t0 = time.perf_counter()
+        qbuf = oracle.fused_quantize_into_fp8(list(tensors), ws, nthreads=nthreads)
+        t1 = time.perf_counter()
+        oracle.fused_reduce_fp8(list(tensors), recv, ws, 3, ReduceOp.AVG, nthreads=nthreads)
+        t2 = time.perf_counter()
+        oracle.fused_dequantize_from_fp8(outs, qbuf, ws, nthreads=nthreads)
+        t3 = time.perf_counter()
+        tq, tr, td = tq + t1 - t0, tr + t2 - t1, td + t3 - t2
+        passes += 1
+    tq, tr, td = tq / passes, tr / passes, td / passes
+    total = sum(ab.values())
+    model = ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {
+        "value": round(total / (tq + tr + td) / 1e9, 3),
+        "unit": "GB/s",
+        "cores": nthreads,
+        "kind": "port",
+        "sample": f"Llama-3-8B layer bucket, {fraction:g} of the rows of each tensor at full row "
+                  f"length, {passes} passes of quantize + reduce (ws=8, AVG) + dequantize, "
+                  f"{(tq + tr + td) * passes:.1f} s of CPU work, mean per pass",
+        "stages_gbs": {"quantize": round(ab["quantize"] / tq / 1e9, 3),
+                       "reduce": round(ab["reduce"] / tr / 1e9, 3),
+                       "dequantize": round(ab["dequantize"] / td / 1e9, 3)},
+        "cpu_model": model,
+    }
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the quantized-collective kernels run on one GPU's share "
+              "and this build has no cross-GPU path; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    from torch.distributed import ReduceOp
+
+    import workloads
+    from torchft_amd import _lib, quantization as q
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a gfx950 GPU", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    rc = _lib.load().tftq_check_device()
+    if rc != 0:
+        print("bench.py: " + _lib.strerror(rc), file=sys.stderr)
+        return 2
+
+    ws, rank, op = 8, args.rank, ReduceOp.AVG
+    dev = "cuda"
+
+    # ---- buffer sets: tensors, received buffer B, gathered buffer G ----------
+    sets = []
+    for k in range(args.sets):
+        slots = []
+        mine = None
+        for peer in range(ws):
+            t = workloads.cfg3(1000 * k + peer, device=dev)
+            qp = q.fused_quantize_into_fp8(t, ws)
+            slot = qp.numel() // ws
+            slots.append(qp[rank * slot:(rank + 1) * slot].clone())
+            if peer == rank:
+                mine = t
+            del t, qp
+        recv = torch.cat(slots)
+        del slots
+        gathered = q.fused_quantize_into_fp8(mine, ws)  # any valid packed buffer of this layout
+        sets.append({"tensors": mine, "recv": recv, "gathered": gathered})
+    torch.cuda.synchronize()
+    ab = workloads.algorithmic_bytes(sets[0]["tensors"], ws)
+
+    # ---- parity gate on the data that is being timed -------------------------
+    from oracle import oracle
+    probe = [sets[0]["tensors"][1]]  # k_proj gradient [1024, 4096]
+    probe_cpu = [probe[0].cpu()]
+    qg = q.fused_quantize_into_fp8(probe, ws)
+    qc = oracle.fused_quantize_into_fp8(list(probe_cpu), ws)
+    ok = torch.equal(qg.cpu(), qc)
+    rg, rcpu = qg.clone(), qc.clone()
+    q.fused_reduce_fp8(probe, rg, ws, rank, op)
+    oracle.fused_reduce_fp8(list(probe_cpu), rcpu, ws, rank, op)
+    ok = ok and torch.equal(rg.cpu(), rcpu)
+    dg, dc = [torch.empty_like(probe[0])], [torch.empty_like(probe_cpu[0])]
+    q.fused_dequantize_from_fp8(dg, qg, ws)
+    oracle.fused_dequantize_from_fp8(dc, qc, ws)
+    ok = ok and torch.equal(dg[0].cpu().view(torch.int16), dc[0].view(torch.int16))
+    if not ok:
+        print("bench.py: GPU results differ from the CPU checker", file=sys.stderr)
+        return 1
+
+    ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
+
+    def step(i, events=None):
+        # the public drop-in functions, exactly as torchft/collectives.py calls them
+        s = sets[i % len(sets)]
+        stream = torch.cuda.current_stream()
+        if events is not None:
+            events[0].record(stream)
+        packed = q.fused_quantize_into_fp8(s["tensors"], ws)
+        if events is not None:
+            events[1].record(stream)
+        q.fused_reduce_fp8(s["tensors"], s["recv"], ws, rank, op)
+        if events is not None:
+            events[2].record(stream)
+        q.fused_dequantize_from_fp8(s["tensors"], s["gathered"], ws)
+        if events is not None:
+            events[3].record(stream)
+        return packed
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    all_events = [[ev() for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, all_events[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    stage_ms = {"quantize": 0.0, "reduce": 0.0, "dequantize": 0.0}
+    for e in all_events:
+        stage_ms["quantize"] += e[0].elapsed_time(e[1])
+        stage_ms["reduce"] += e[1].elapsed_time(e[2])
+        stage_ms["dequantize"] += e[2].elapsed_time(e[3])
+    for k in stage_ms:
+        stage_ms[k] /= args.steps
+    total_bytes = sum(ab.values())
+    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+
+    stages = {}
+    for k in stage_ms:
+        gbs = ab[k] / (stage_ms[k] * 1e-3) / 1e9
+        stages[k] = {"us": round(stage_ms[k] * 1e3, 2), "bytes": ab[k], "GBs": round(gbs, 1),
+                     "frac": round(gbs / HBM_PEAK_GBS, 4)}
+
+    out = {
+        "metric": "quantize+reduce+dequant HBM GB/s on 1 MI355X",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 3: Llama-3-8B decoder-layer gradient bucket, "
+                               "9 bf16 tensors, 218112000 elements, ws=8, reduce AVG, rank "
+                               f"{rank}; {len(sets)} rotating buffer sets (cold last-level cache)",
+                   "input_dtype": "bf16", "packed_bytes": int(sets[0]["gathered"].numel()),
+                   "algorithmic_bytes_per_step": total_bytes},
+        "roofline": {"bound": "hbm", "kernel": "k_quantize<bf16>",
+                     "achieved": stages["quantize"]["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": stages["quantize"]["frac"], "traffic": None},
+        "stages": stages,
+        "parity": "quantize, reduce, dequantize byte-identical to the CPU checker on the probe tensor",
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_rows)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

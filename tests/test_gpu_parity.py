@@ -286,9 +286,15 @@ def test_cfg3_full_size(q, oracle):
     for x, o in zip(peers_gpu[0], outs):
         xf, of = x.float().view(x.shape[0], -1), o.float().view(x.shape[0], -1)
         amax = xf.abs().amax(dim=1, keepdim=True)
-        # fp8 half-ULP (2^-4 relative, 2^-10/s absolute) plus the bf16 store rounding (2^-9)
-        tol = torch.maximum(xf.abs() * (2 ** -4 + 2 ** -8), amax * (2 ** -10 / 448.0) * 1.01)
-        assert ((xf - of).abs() <= tol).all()
+        # fp8 half-ULP (2^-4 relative for normal codes, 2^-10 / s absolute for subnormal
+        # ones) plus the bf16 store rounding (half a bf16 ULP of the output, 2^-8 relative)
+        tol = torch.maximum(xf.abs() * 2 ** -4, amax * (2 ** -10 / 448.0)) * 1.001 + of.abs() * 2 ** -8
+        bad = (xf - of).abs() > tol
+        if bad.any():
+            r, c = bad.nonzero()[0].tolist()
+            raise AssertionError(
+                f"round trip out of tolerance in {tuple(x.shape)}: {int(bad.sum())} elements, first at "
+                f"({r},{c}): x={xf[r, c].item()!r} out={of[r, c].item()!r} amax={amax[r].item()!r}")
     # idempotence: quantizing the dequantized tensors reproduces the codes (scales may move an ulp)
     q2 = q.fused_quantize_into_fp8(list(outs), ws)
     d2 = [torch.empty_like(t) for t in outs]
