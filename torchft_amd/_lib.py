@@ -43,7 +43,8 @@ SYMBOLS = [
 
 
 def lib_path() -> str:
-    return _build.LIB_PATH
+    """Path of the shared library; ``TFTQ_LIB`` overrides the in-tree build."""
+    return os.environ.get("TFTQ_LIB") or _build.LIB_PATH
 
 
 def load() -> ctypes.CDLL:

@@ -49,7 +49,7 @@ struct Seg {
     int32_t row_bytes;   // 4 + round_up(n, 4)
     int32_t wg_begin[3]; // first workgroup of this segment, per stage
     uint8_t kind[3];     // lane mapping, per stage
-    uint8_t pad;
+    uint8_t reduce_rows_per_team;  // reduce: consecutive rows one team works through (wide teams)
 };
 static_assert(sizeof(Seg) == 64, "Seg must be 64 bytes");
 
@@ -66,6 +66,7 @@ struct tftq_plan {
     int64_t output_size;
     int64_t max_rows;
     int32_t nwg[3];
+    int32_t xcd_begin[3][9];  // per stage: first workgroup of each XCD's share, balanced by bytes
     std::vector<Seg> segs;
     const void *device_table;  // set by the caller when nseg > TFTQ_N_INLINE
 };
@@ -79,6 +80,7 @@ struct KParams {
     int32_t nwg;
     int32_t ws;
     int32_t rank;
+    int32_t xcd_begin[9];  // workgroups [xcd_begin[x], xcd_begin[x+1]) run on XCD x
     int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG general
     float div;          // reduce: 1.0 or float(ws)
     float inv_div;      // reduce: exact reciprocal when div_mode == 1

@@ -27,6 +27,9 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
+
+#include <algorithm>
 
 #include "../../include/tftq.h"
 #include "tftq_internal.h"
@@ -44,6 +47,14 @@ struct bf16_tag {};
 struct f16_tag {};
 
 #define DEV __device__ __forceinline__
+// Streaming accesses for data that is touched once per kernel.
+#ifdef TFTQ_NO_NT
+#define LOAD_STREAM(ptr) (*(ptr))
+#define STORE_STREAM(val, ptr) (*(ptr) = (val))
+#else
+#define LOAD_STREAM(ptr) __builtin_nontemporal_load(ptr)
+#define STORE_STREAM(val, ptr) __builtin_nontemporal_store((val), (ptr))
+#endif
 #define GLOBAL __attribute__((address_space(1)))
 
 // Tensor addresses arrive as integers; tell the compiler they are global
@@ -257,14 +268,15 @@ template <> struct Elem<f16_tag> {
 // ---------------------------------------------------------------------------
 // workgroup -> (segment, first row)
 // ---------------------------------------------------------------------------
-// Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  Give XCD x
-// the x-th contiguous eighth of the work instead.  The grid is launched with
-// 8 * ceil(nwg / 8) workgroups; ids that map past nwg return -1.
-DEV int virtual_block(int nwg)
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  XCD x works on
+// the contiguous range [xcd_begin[x], xcd_begin[x+1]) instead (ranges balanced by
+// bytes on the host).  The grid has 8 * (longest range) workgroups; ids past
+// the end of their range return -1.
+DEV int virtual_block(const KParams &p)
 {
-    const int per_xcd = (nwg + 7) >> 3;
-    const int vb = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    return vb < nwg ? vb : -1;
+    const int x = (int)(blockIdx.x & 7);
+    const int vb = p.xcd_begin[x] + (int)(blockIdx.x >> 3);
+    return vb < p.xcd_begin[x + 1] ? vb : -1;
 }
 
 template <bool INLINE, int STAGE>
@@ -319,13 +331,16 @@ DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
         u32x2 o;
         o.x = pack_fp8x4(f[0] * s, f[1] * s, f[2] * s, f[3] * s);
         o.y = pack_fp8x4(f[4] * s, f[5] * s, f[6] * s, f[7] * s);
-        *(GLOBAL u32x2_a4 *)(payload + 2 * idx) = o;
+        *(GLOBAL u32x2_a4 *)(payload + 2 * idx) = o;  // plain store: rows start 4 bytes off a line, L2 merges
     }
 }
 
-// Contiguous, 16-byte aligned rows of at most TEAM * QV vectors.
-template <typename T, int TEAM>
-DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds)
+// Contiguous, 16-byte aligned rows of at most TEAM * KMAX vectors.  The KMAX
+// loads of a lane are issued back to back without a branch in between: lanes
+// past the end of the row re-read its last vector (a duplicate cannot change
+// the maximum) and simply do not store.
+template <typename T, int TEAM, int KMAX>
+DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float *lds)
 {
     const bool active = row < s.slice_rows * p.ws;
     GLOBAL u32 *out = as_global<u32>(p.packed + (active ? row_addr(s, p.slot_size, row) : 0));
@@ -338,24 +353,28 @@ DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *
     constexpr int EPV = Elem<T>::EPV;
     const int nvec = s.n / EPV;
     GLOBAL const u32x4 *in = as_global<const u32x4>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
-    u32x4 v[QV];
+    u32x4 v[KMAX];
 #pragma unroll
-    for (int k = 0; k < QV; k++) {
-        const int idx = k * TEAM + lane;
-        const u32x4 z = {0, 0, 0, 0};
-        v[k] = idx < nvec ? __builtin_nontemporal_load(in + idx) : z;
-    }
+    for (int k = 0; k < KMAX; k++) v[k] = LOAD_STREAM(in + min(k * TEAM + lane, nvec - 1));
     float amax = 0.0f;
 #pragma unroll
-    for (int k = 0; k < QV; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+    for (int k = 0; k < KMAX; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
     amax = team_max<TEAM>(amax, lds);
     const float sc = calc_scale(amax);
     if (lane == 0) out[0] = as_u(sc);
 #pragma unroll
-    for (int k = 0; k < QV; k++) {
+    for (int k = 0; k < KMAX; k++) {
         const int idx = k * TEAM + lane;
         if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
     }
+}
+
+template <typename T, int TEAM>
+DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds)
+{
+    // same branch for the whole workgroup
+    if (s.n / Elem<T>::EPV <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
+    else quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
 }
 
 // Any strides, any alignment, any n: element loads, two passes over the row
@@ -398,7 +417,7 @@ template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
-    const int vb = virtual_block(p.nwg);
+    const int vb = virtual_block(p);
     if (vb < 0) return;
     const Seg s = find_seg<INLINE, ST_Q>(p, inl, vb);
     const int blk = vb - s.wg_begin[ST_Q];
@@ -421,30 +440,6 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
 // ---------------------------------------------------------------------------
 // dequantize
 // ---------------------------------------------------------------------------
-template <typename T>
-DEV u32x4 dequant_vec_unit(GLOBAL const u32 *payload, int idx, float r, float r_lo)
-{
-    constexpr int EPV = Elem<T>::EPV;
-    float o[EPV];
-    if constexpr (EPV == 4) {
-        float f[4];
-        unpack_fp8x4(payload[idx], f);
-#pragma unroll
-        for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], r, r_lo);
-    } else {
-        const u32x2 w = *(GLOBAL const u32x2_a4 *)(payload + 2 * idx);
-        float f[4], g[4];
-        unpack_fp8x4(w.x, f);
-        unpack_fp8x4(w.y, g);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            o[e] = div_fast_signed(f[e], r, r_lo);
-            o[4 + e] = div_fast_signed(g[e], r, r_lo);
-        }
-    }
-    return Elem<T>::pack(o);
-}
-
 // Any strides; also the path of rows whose scale is outside the range of the
 // fast exact division (plain IEEE divide, one element per lane and step).
 template <typename T, int TEAM>
@@ -469,6 +464,9 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
+// Contiguous, 16-byte aligned rows.  Four vectors per lane and step; their loads
+// are issued together without a branch (lanes past the end re-read the last
+// vector and do not store).
 template <typename T, int TEAM>
 DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
 {
@@ -479,17 +477,44 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
         dequantize_gen<T, TEAM>(s, p, row, lane);
         return;
     }
-    const int nvec = s.n / Elem<T>::EPV;
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int DV = 4;
+    const int nvec = s.n / EPV;
     GLOBAL u32x4 *out = as_global<u32x4>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
-#pragma unroll 4
-    for (int idx = lane; idx < nvec; idx += TEAM)
-        out[idx] = dequant_vec_unit<T>(in + 1, idx, c.r, c.r_lo);
+    for (int base = 0; base < nvec; base += DV * TEAM) {
+        u32x2 w[DV];
+#pragma unroll
+        for (int k = 0; k < DV; k++) {
+            const int idx = min(base + k * TEAM + lane, nvec - 1);
+            if constexpr (EPV == 4) {
+                w[k].x = LOAD_STREAM(in + 1 + idx);
+                w[k].y = 0;
+            } else {
+                w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < DV; k++) {
+            const int idx = base + k * TEAM + lane;
+            float o[EPV];
+            float f[4];
+            unpack_fp8x4(w[k].x, f);
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], c.r, c.r_lo);
+            if constexpr (EPV == 8) {
+                unpack_fp8x4(w[k].y, f);
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(f[e], c.r, c.r_lo);
+            }
+            if (idx < nvec) STORE_STREAM(Elem<T>::pack(o), out + idx);
+        }
+    }
 }
 
 template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const InlineTable inl)
 {
-    const int vb = virtual_block(p.nwg);
+    const int vb = virtual_block(p);
     if (vb < 0) return;
     const Seg s = find_seg<INLINE, ST_D>(p, inl, vb);
     const int blk = vb - s.wg_begin[ST_D];
@@ -553,6 +578,7 @@ DEV void store_codes(GLOBAL u32 *payload, int d0, int ndw, const u32x4 w)
 DEV void accumulate16(float (&acc)[16], const u32x4 w, float r, float r_lo)
 {
     const u32 ww[4] = {w.x, w.y, w.z, w.w};
+
 #pragma unroll
     for (int t = 0; t < 4; t++) {
         float f[4];
@@ -590,6 +616,7 @@ DEV GLOBAL const u32 *peer_row(const KParams &p, int k, int64_t off)
 {
     int peer = p.rank + k;  // :407
     if (peer >= p.ws) peer -= p.ws;
+
     return as_global<const u32>(p.packed + (int64_t)peer * p.slot_size + off);
 }
 
@@ -650,21 +677,6 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
     const int wlane = threadIdx.x & 63;
 
-    // can every peer's scale take the fast exact division?
-    bool all_fast = true;
-    if (TEAM >= 64) {
-        for (int k = wlane; k < p.ws; k += 64)
-            all_fast = all_fast && scale_is_fast(guarded_scale(peer_row(p, k, off)));
-        all_fast = __builtin_amdgcn_ballot_w64(!all_fast) == 0;
-    } else {
-        for (int k = 0; k < p.ws; k++)
-            all_fast = all_fast && scale_is_fast(guarded_scale(peer_row(p, k, off)));
-    }
-    if (!all_fast) {
-        reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);
-        return;
-    }
-
     float acc[UNITS][16];
 #pragma unroll
     for (int u = 0; u < UNITS; u++)
@@ -672,17 +684,16 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
         for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
 
     for (int kc = 0; kc < p.ws; kc += 64) {
-        // wide teams: lane l of every wavefront prepares peer kc + l
-        float cr = 1.0f, cl = 0.0f;
-        if (TEAM >= 64 && kc + wlane < p.ws) {
-            const DivCoef c = make_div(guarded_scale(peer_row(p, kc + wlane, off)));
-            cr = c.r;
-            cl = c.r_lo;
-        }
         const int kend = min(p.ws, kc + 64);
-        for (int k0 = kc; k0 < kend; k0 += PB) {
-            u32x4 w[PB][UNITS];
-            float sraw[PB];
+        // Wide teams: lane l of every wavefront fetches the scale of peer kc + l
+        // first, then the codes of the first peers go in flight, and only then
+        // are the scales turned into division coefficients.
+        float my_scale = 1.0f;
+        if (TEAM >= 64 && kc + wlane < p.ws) my_scale = guarded_scale(peer_row(p, kc + wlane, off));
+
+        u32x4 w[PB][UNITS];
+        float sraw[PB];
+        auto load_batch = [&](int k0) {
 #pragma unroll
             for (int b = 0; b < PB; b++) {
                 if (k0 + b < kend) {
@@ -691,6 +702,31 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 #pragma unroll
                     for (int u = 0; u < UNITS; u++)
                         w[b][u] = load_codes(prow + 1, (u * TEAM + lane) * 4, ndw, n);
+                }
+            }
+        };
+        load_batch(kc);
+
+        float cr = 1.0f, cl = 0.0f;
+        if (TEAM >= 64) {
+            const DivCoef c = make_div(my_scale);
+            cr = c.r;
+            cl = c.r_lo;
+            if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // some peer needs the plain divide
+                reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);
+                return;
+            }
+        }
+        for (int k0 = kc; k0 < kend; k0 += PB) {
+            if (k0 != kc) load_batch(k0);
+            if (TEAM < 64) {
+                bool fast = true;
+#pragma unroll
+                for (int b = 0; b < PB; b++)
+                    if (k0 + b < kend) fast = fast && scale_is_fast(sraw[b]);
+                if (!fast) {  // same decision in every lane of the team
+                    reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);
+                    return;
                 }
             }
 #pragma unroll
@@ -729,25 +765,181 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
     if (lane == 0) orow[0] = as_u(s2);  // :375
 }
 
+// Several rows per team, software-pipelined: the codes of the next batch of
+// peers (of this row or of the next row) are in flight while the current batch
+// is accumulated, so a wavefront always has loads outstanding.  A batch is
+// R_VPB 16-byte vectors per lane: R_VPB / UNITS peers of one row.  Loads carry
+// no branch: a lane past the end of the row re-reads the row's last vector, a
+// batch past the last peer re-reads the last peer, and both are ignored later.
+// Needs TEAM >= 64 (a peer's scale lives in one lane of each wavefront),
+// ws <= 64 and rows that are a whole number (>= 1) of 16-byte vectors.
+#ifndef TFTQ_R_VPB
+#define TFTQ_R_VPB 4
+#endif
+
+template <int TEAM, int UNITS, bool PIPE, bool GDIV>
+DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane, float *lds)
+{
+    constexpr int PB = TFTQ_R_VPB / UNITS >= 1 ? TFTQ_R_VPB / UNITS : 1;  // peers per batch
+    if (nrows <= 0) return;
+    const int nvec = ((s.row_bytes >> 2) - 1) >> 2;
+    const int ws = p.ws;
+    const int nb = (ws + PB - 1) / PB;  // batches per row
+    const int total = nrows * nb;
+    const int wlane = threadIdx.x & 63;
+    const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
+
+    int vidx[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) vidx[u] = min(u * TEAM + lane, nvec - 1);
+
+    struct Batch {
+        u32x4 w[PB][UNITS];
+        float scale;  // lane l: guarded scale of peer min(l, ws-1) of the batch's row
+    };
+    Batch A, B;
+
+    int lrow = 0, lbatch = 0;  // next batch to load
+    auto issue = [&](Batch &dst) {
+        const int64_t off = s.slot_off + (int64_t)(j0 + lrow) * s.row_bytes;
+        dst.scale = as_f(peer_row(p, speer, off)[0]);
+#pragma unroll
+        for (int b = 0; b < PB; b++) {
+            GLOBAL const u32x4_a4 *pv =
+                (GLOBAL const u32x4_a4 *)(peer_row(p, min(lbatch * PB + b, ws - 1), off) + 1);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) dst.w[b][u] = LOAD_STREAM(pv + vidx[u]);
+        }
+        if (++lbatch == nb) {
+            lbatch = 0;
+            ++lrow;
+        }
+    };
+
+    float acc[UNITS][16];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+    int crow = 0, cbatch = 0;  // batch being consumed
+    float cr = 1.0f, cl = 0.0f;
+    bool row_fast = true;
+
+    auto consume = [&](const Batch &src) {
+        if (cbatch == 0) {
+            const float sc = src.scale == 0.0f ? 1.0f : src.scale;  // padding rows (:419)
+            const DivCoef c = make_div(sc);
+            cr = c.r;
+            cl = c.r_lo;
+            row_fast = __builtin_amdgcn_ballot_w64(!c.fast) == 0;  // same in all wavefronts of the team
+        }
+        if (row_fast) {
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                const int k = cbatch * PB + b;
+                if (k < ws) {
+                    const float pr = bcast_lane(cr, k), pl = bcast_lane(cl, k);
+#pragma unroll
+                    for (int u = 0; u < UNITS; u++) accumulate16(acc[u], src.w[b][u], pr, pl);
+                }
+            }
+        }
+        if (++cbatch == nb) {
+            const int j = j0 + crow;
+            if (row_fast) {
+                float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
+#pragma unroll
+                for (int u = 0; u < UNITS; u++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+                amax = team_max<TEAM>(amax, lds);
+                const float s2 = calc_scale(amax / p.div);  // :340
+                const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+                GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+#pragma unroll
+                for (int u = 0; u < UNITS; u++) {
+                    const u32x4 o = requant16<GDIV>(acc[u], s2, p);
+                    if (u * TEAM + lane < nvec) ((GLOBAL u32x4_a4 *)(orow + 1))[u * TEAM + lane] = o;
+                }
+                if (lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+            } else {
+                reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
+            }
+#pragma unroll
+            for (int u = 0; u < UNITS; u++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+            cbatch = 0;
+            ++crow;
+        }
+    };
+
+    if (!PIPE) {  // long rows: one batch in flight keeps the register count down
+        for (int i = 0; i < total; i++) {
+            issue(A);
+            consume(A);
+        }
+        return;
+    }
+    issue(A);
+    int i = 0;
+    for (; i + 2 < total; i += 2) {
+        issue(B);
+        consume(A);
+        issue(A);
+        consume(B);
+    }
+    if (i + 1 < total) {
+        issue(B);
+        consume(A);
+        consume(B);
+    } else {
+        consume(A);
+    }
+}
+
+#ifndef TFTQ_R_MINWAVES
+#define TFTQ_R_MINWAVES 1
+#endif
 template <bool INLINE, bool GDIV>
-__global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
+__global__ __launch_bounds__(TFTQ_WG, TFTQ_R_MINWAVES) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
-    const int vb = virtual_block(p.nwg);
+    const int vb = virtual_block(p);
     if (vb < 0) return;
     const Seg s = find_seg<INLINE, ST_R>(p, inl, vb);
     const int blk = vb - s.wg_begin[ST_R];
     const int tid = threadIdx.x;
     const int ndw = (s.row_bytes >> 2) - 1;
+    const int rpt = s.reduce_rows_per_team;
     switch (s.kind[ST_R]) {
-    case K_GEN256:
-        if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, blk, tid, lds);
-        else if (ndw <= 4096) reduce_row<256, 4, GDIV>(s, p, blk, tid, lds);
-        else reduce_row_slow<256, GDIV>(s, p, blk, tid, lds);
+    case K_GEN256: {
+        const int j0 = blk * rpt;
+        const int nrows = min(rpt, s.slice_rows - j0);
+        if (ndw > 4096) {
+            for (int r = 0; r < nrows; r++) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
+        } else if (p.ws > 64 || (ndw & 3) != 0) {
+            for (int r = 0; r < nrows; r++) {
+                if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j0 + r, tid, lds);
+                else reduce_row<256, 4, GDIV>(s, p, j0 + r, tid, lds);
+            }
+        } else if (ndw <= 1024) {
+            reduce_rows<256, 1, true, GDIV>(s, p, j0, nrows, tid, lds);
+        } else {
+            reduce_rows<256, 4, false, GDIV>(s, p, j0, nrows, tid, lds);
+        }
         break;
-    case K_GEN64:
-        reduce_row<64, 1, GDIV>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds);
+    }
+    case K_GEN64: {
+        const int j0 = (blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6)) * rpt;
+        const int nrows = min(rpt, s.slice_rows - j0);
+        if (p.ws > 64 || (ndw & 3) != 0) {
+            for (int r = 0; r < nrows; r++) reduce_row<64, 1, GDIV>(s, p, j0 + r, tid & 63, lds);
+        } else {
+            reduce_rows<64, 1, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
+        }
         break;
+    }
     case K_GEN8: reduce_row<8, 1, GDIV>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
     case K_GEN1: reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds); break;
     default: break;
@@ -771,6 +963,27 @@ extern "C" int tftq_check_device(void)
                : TFTQ_E_ARCH;
 }
 
+// TFTQ_XCD_MODE (tuning aid): 0 = equal workgroup counts per XCD, 1 = equal bytes (default)
+static int xcd_mode()
+{
+    static const int mode = [] {
+        const char *e = getenv("TFTQ_XCD_MODE");
+        return e ? atoi(e) : 1;
+    }();
+    return mode;
+}
+
+static void xcd_ranges(const tftq_plan *plan, int stage, KParams *kp)
+{
+    const int nwg = plan->nwg[stage];
+    if (xcd_mode() == 0) {
+        const int per = (nwg + 7) / 8;
+        for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = std::min(nwg, x * per);
+    } else {
+        for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = plan->xcd_begin[stage][x];
+    }
+}
+
 static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t packed_bytes,
                        KParams *kp, InlineTable *inl, bool *use_inline)
 {
@@ -785,6 +998,7 @@ static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t p
     kp->nseg = plan->nseg;
     kp->nwg = plan->nwg[stage];
     kp->ws = plan->ws;
+    xcd_ranges(plan, stage, kp);
     kp->rank = 0;
     kp->div_mode = 0;
     kp->div = 1.0f;
@@ -794,15 +1008,20 @@ static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t p
     return 0;
 }
 
-static inline unsigned grid_of(int nwg) { return (unsigned)(((nwg + 7) / 8) * 8); }
+static inline unsigned grid_of(const KParams &kp)
+{
+    int longest = 0;
+    for (int x = 0; x < 8; x++) longest = std::max(longest, kp.xcd_begin[x + 1] - kp.xcd_begin[x]);
+    return (unsigned)(8 * longest);
+}
 
 template <typename T>
 static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, hipStream_t st)
 {
     if (use_inline)
-        hipLaunchKernelGGL((k_quantize<T, true>), dim3(grid_of(kp.nwg)), dim3(TFTQ_WG), 0, st, kp, inl);
+        hipLaunchKernelGGL((k_quantize<T, true>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
     else
-        hipLaunchKernelGGL((k_quantize<T, false>), dim3(grid_of(kp.nwg)), dim3(TFTQ_WG), 0, st, kp, inl);
+        hipLaunchKernelGGL((k_quantize<T, false>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
     return (int)hipGetLastError();
 }
 
@@ -810,9 +1029,9 @@ template <typename T>
 static int launch_d(const KParams &kp, const InlineTable &inl, bool use_inline, hipStream_t st)
 {
     if (use_inline)
-        hipLaunchKernelGGL((k_dequantize<T, true>), dim3(grid_of(kp.nwg)), dim3(TFTQ_WG), 0, st, kp, inl);
+        hipLaunchKernelGGL((k_dequantize<T, true>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
     else
-        hipLaunchKernelGGL((k_dequantize<T, false>), dim3(grid_of(kp.nwg)), dim3(TFTQ_WG), 0, st, kp, inl);
+        hipLaunchKernelGGL((k_dequantize<T, false>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
     return (int)hipGetLastError();
 }
 
@@ -879,7 +1098,7 @@ extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_b
     }
     if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid(grid_of(kp.nwg)), block(TFTQ_WG);
+    const dim3 grid(grid_of(kp)), block(TFTQ_WG);
     if (kp.div_mode == 2) {
         if (use_inline) hipLaunchKernelGGL((k_reduce<true, true>), grid, block, 0, st, kp, inl);
         else hipLaunchKernelGGL((k_reduce<false, true>), grid, block, 0, st, kp, inl);

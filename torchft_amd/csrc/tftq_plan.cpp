@@ -6,6 +6,7 @@
 // the reference keeps them in int32 (:514-515).
 
 #include <limits.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <new>
@@ -77,6 +78,80 @@ static uint8_t pick_reduce_kind(const Seg &s)
     return K_GEN256;
 }
 
+// Reduce: a wide team works through several consecutive rows so that it can
+// prefetch the next one; aim at about TFTQ_R_TEAM_BYTES of peer rows per team.
+static int reduce_team_bytes()
+{
+    static const int v = [] {
+        const char *e = getenv("TFTQ_R_TEAM_BYTES");
+        return e ? atoi(e) : 32 * 1024;
+    }();
+    return v;
+}
+
+static int pick_reduce_rows(const Seg &s, int ws)
+{
+    if (s.kind[ST_R] != K_GEN256 && s.kind[ST_R] != K_GEN64) return 1;
+    const int64_t per_row = (int64_t)s.row_bytes * ws;
+    int64_t r = (reduce_team_bytes() + per_row / 2) / per_row;
+    if (r < 1) r = 1;
+    if (r > 16) r = 16;
+    return (int)r;
+}
+
+static int rows_per_wg_of(const Seg &s, int st)
+{
+    const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
+    return st == ST_R ? teams * s.reduce_rows_per_team : teams;
+}
+
+// Bytes one workgroup of segment s moves in a stage.
+static double wg_weight(const Seg &s, int st, int esz, int ws)
+{
+    const double rows = (double)rows_per_wg_of(s, st);
+    if (st == ST_R) return rows * (double)s.row_bytes * (ws + 1);
+    return rows * ((double)s.n * esz + (double)s.row_bytes);
+}
+
+// Workgroup ids are dealt round-robin to the 8 XCDs by the hardware; the
+// kernels turn that into one contiguous range of workgroups per XCD.  Choose
+// the ranges so that every XCD moves about the same number of bytes (rows of
+// different tensors differ in length by up to 3.5x in one call).
+static void balance_xcds(tftq_plan *p)
+{
+    for (int st = 0; st < 3; st++) {
+        int32_t *xb = p->xcd_begin[st];
+        const int nwg = p->nwg[st];
+        double total = 0;
+        for (int i = 0; i < p->nseg; i++) {
+            const Seg &s = p->segs[(size_t)i];
+            const int end = i + 1 < p->nseg ? p->segs[(size_t)i + 1].wg_begin[st] : nwg;
+            total += (double)(end - s.wg_begin[st]) * wg_weight(s, st, p->esz, p->ws);
+        }
+        xb[0] = 0;
+        int x = 1;
+        double cum = 0;
+        for (int i = 0; i < p->nseg && x < 8; i++) {
+            const Seg &s = p->segs[(size_t)i];
+            const int begin = s.wg_begin[st];
+            const int end = i + 1 < p->nseg ? p->segs[(size_t)i + 1].wg_begin[st] : nwg;
+            const double w = wg_weight(s, st, p->esz, p->ws);
+            if (end == begin || w <= 0) continue;
+            const double seg_total = (double)(end - begin) * w;
+            while (x < 8 && cum + seg_total >= total * x / 8.0) {
+                double k = (total * x / 8.0 - cum) / w;  // workgroups of this segment before the cut
+                int cut = begin + (int)(k + 0.5);
+                if (cut < xb[x - 1]) cut = xb[x - 1];
+                if (cut > end) cut = end;
+                xb[x++] = cut;
+            }
+            cum += seg_total;
+        }
+        while (x <= 8) xb[x++] = nwg;
+        xb[8] = nwg;
+    }
+}
+
 extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
                                 const int64_t *shapes, const int64_t *strides, int ws,
                                 tftq_plan **out)
@@ -123,10 +198,11 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
 
         s.kind[ST_Q] = s.kind[ST_D] = pick_io_kind(s, p->esz);
         s.kind[ST_R] = pick_reduce_kind(s);
+        s.reduce_rows_per_team = (uint8_t)pick_reduce_rows(s, ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
             s.wg_begin[st] = (int32_t)wg[st];
-            const int rows_per_wg = TFTQ_WG / tftq_team_of(s.kind[st]);
+            const int rows_per_wg = rows_per_wg_of(s, st);
             wg[st] += cdiv64(rows[st], rows_per_wg);
             if (wg[st] > INT32_MAX - 16) {
                 delete p;
@@ -135,6 +211,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         }
     }
     for (int st = 0; st < 3; st++) p->nwg[st] = (int32_t)wg[st];
+    balance_xcds(p);
     *out = p;
     return 0;
 }
