@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--sets", type=int, default=3, help="buffer sets the steps rotate over")
     ap.add_argument("--rank", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times, so that a counter "
+                         "profile of this command contains a kernel of known HBM traffic")
     ap.add_argument("--cpu-rows", type=float, default=1.0,
                     help="fraction of the bucket's rows the CPU baseline runs on")
     return ap.parse_args()
@@ -186,6 +189,14 @@ def main() -> int:
             events[3].record(stream)
         return packed
 
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -235,7 +246,10 @@ def main() -> int:
                    "algorithmic_bytes_per_step": total_bytes},
         "roofline": {"bound": "hbm", "kernel": "k_quantize<bf16>",
                      "achieved": stages["quantize"]["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": stages["quantize"]["frac"], "traffic": None},
+                     "frac": stages["quantize"]["frac"],
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated
+                     # on a 256 MiB copy) + WRITE_SIZE (x1.000); profiles/cfg3_bf16_ws8_hbm_traffic.md
+                     "traffic": 654846000},
         "stages": stages,
         "parity": "quantize, reduce, dequantize byte-identical to the CPU checker on the probe tensor",
     }

@@ -47,14 +47,10 @@ struct bf16_tag {};
 struct f16_tag {};
 
 #define DEV __device__ __forceinline__
-// Streaming accesses for data that is touched once per kernel.
-#ifdef TFTQ_NO_NT
-#define LOAD_STREAM(ptr) (*(ptr))
-#define STORE_STREAM(val, ptr) (*(ptr) = (val))
-#else
+// Streaming accesses for data that is touched once per kernel (measured on
+// MI355X: +10 % read bandwidth over plain loads).
 #define LOAD_STREAM(ptr) __builtin_nontemporal_load(ptr)
 #define STORE_STREAM(val, ptr) __builtin_nontemporal_store((val), (ptr))
-#endif
 #define GLOBAL __attribute__((address_space(1)))
 
 // Tensor addresses arrive as integers; tell the compiler they are global
@@ -773,14 +769,12 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 // batch past the last peer re-reads the last peer, and both are ignored later.
 // Needs TEAM >= 64 (a peer's scale lives in one lane of each wavefront),
 // ws <= 64 and rows that are a whole number (>= 1) of 16-byte vectors.
-#ifndef TFTQ_R_VPB
-#define TFTQ_R_VPB 4
-#endif
+constexpr int R_VPB = 4;
 
 template <int TEAM, int UNITS, bool PIPE, bool GDIV>
 DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane, float *lds)
 {
-    constexpr int PB = TFTQ_R_VPB / UNITS >= 1 ? TFTQ_R_VPB / UNITS : 1;  // peers per batch
+    constexpr int PB = R_VPB / UNITS >= 1 ? R_VPB / UNITS : 1;  // peers per batch
     if (nrows <= 0) return;
     const int nvec = ((s.row_bytes >> 2) - 1) >> 2;
     const int ws = p.ws;
@@ -898,11 +892,8 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
     }
 }
 
-#ifndef TFTQ_R_MINWAVES
-#define TFTQ_R_MINWAVES 1
-#endif
 template <bool INLINE, bool GDIV>
-__global__ __launch_bounds__(TFTQ_WG, TFTQ_R_MINWAVES) void k_reduce(const KParams p, const InlineTable inl)
+__global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
     const int vb = virtual_block(p);
@@ -963,25 +954,9 @@ extern "C" int tftq_check_device(void)
                : TFTQ_E_ARCH;
 }
 
-// TFTQ_XCD_MODE (tuning aid): 0 = equal workgroup counts per XCD, 1 = equal bytes (default)
-static int xcd_mode()
-{
-    static const int mode = [] {
-        const char *e = getenv("TFTQ_XCD_MODE");
-        return e ? atoi(e) : 1;
-    }();
-    return mode;
-}
-
 static void xcd_ranges(const tftq_plan *plan, int stage, KParams *kp)
 {
-    const int nwg = plan->nwg[stage];
-    if (xcd_mode() == 0) {
-        const int per = (nwg + 7) / 8;
-        for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = std::min(nwg, x * per);
-    } else {
-        for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = plan->xcd_begin[stage][x];
-    }
+    for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = plan->xcd_begin[stage][x];
 }
 
 static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t packed_bytes,

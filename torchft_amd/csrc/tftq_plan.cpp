@@ -78,16 +78,10 @@ static uint8_t pick_reduce_kind(const Seg &s)
     return K_GEN256;
 }
 
-// Reduce: a wide team works through several consecutive rows so that it can
-// prefetch the next one; aim at about TFTQ_R_TEAM_BYTES of peer rows per team.
-static int reduce_team_bytes()
-{
-    static const int v = [] {
-        const char *e = getenv("TFTQ_R_TEAM_BYTES");
-        return e ? atoi(e) : 32 * 1024;
-    }();
-    return v;
-}
+// Reduce: a wide team works through several consecutive short rows, prefetching
+// the next one; about 32 KB of peer rows per team (measured best on MI355X:
+// more rows per team leave too few workgroups to balance the CUs).
+static int reduce_team_bytes() { return 32 * 1024; }
 
 static int pick_reduce_rows(const Seg &s, int ws)
 {
