@@ -11,7 +11,7 @@ the same GPU from 8 independently seeded peers.  Inputs are resident in HBM
 before the timed region.  The step rotates over several buffer sets so that the
 256 MB last-level cache cannot hold the working set of the next step ("cold").
 
-Workload: BASELINE configuration 3, the Llama-3-8B decoder-layer gradient
+Workload: benchmark configuration 3, the Llama-3-8B decoder-layer gradient
 bucket (9 bf16 tensors, 218 112 000 elements, per-row std log-uniform in
 [1e-5, 1e-1]), world size 8, reduce op AVG.
 

@@ -128,7 +128,7 @@ def test_golden_vectors_gpu(q):
             assert bytes(o.cpu().contiguous().view(torch.uint8).flatten().tolist()).hex() == h
 
 
-# ---- BASELINE configurations ---------------------------------------------------
+# ---- the five benchmark configurations ---------------------------------------------------
 def test_cfg1_cpu_plumbing_shapes(q, oracle):
     peers = [workloads.cfg1(s) for s in (0, 1)]
     outs = full_check(q, oracle, peers, 2, ReduceOp.SUM)

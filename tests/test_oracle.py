@@ -42,7 +42,7 @@ def from_hex(h, dtype=torch.uint8):
 def test_layout_worked_examples(oracle):
     assert oracle.layout([(256, 512), (1024, 1)], 2) == ([0, 66048], 70144, 140288)
     assert oracle.layout([(5, 3), (1, 7)], 4) == ([0, 16], 28, 112)
-    # BASELINE configurations 2 and 3
+    # benchmark configurations 2, 3 and 4
     assert oracle.layout([(4096, 4096)], 8)[1:] == (2099200, 16793600)
     shp = [s if len(s) == 2 else (s[0], 1) for _, s in workloads.LLAMA3_8B_LAYER]
     assert oracle.layout(shp, 8)[1:] == (27292672, 218341376)
@@ -246,7 +246,7 @@ def test_c_vs_torch_restatement_strided(oracle):
 
 
 def test_cfg1_plumbing(oracle):
-    """BASELINE configuration 1, end to end on the CPU checker."""
+    """Benchmark configuration 1 (two fp32 tensors, 2 peers, SUM), end to end on the CPU checker."""
     peers = [workloads.cfg1(s) for s in (0, 1)]
     qs = [oracle.fused_quantize_into_fp8(list(t), 2) for t in peers]
     assert qs[0].numel() == 140288
