@@ -7,7 +7,18 @@ from .quantization import (  # noqa: F401
     fused_reduce_fp8,
 )
 
+from .collectives import (  # noqa: F401
+    allocate_reduce_scatter_output,
+    allreduce_quantized,
+    get_padded_sizes,
+    reduce_scatter_quantized,
+)
+
 __all__ = [
+    "allocate_reduce_scatter_output",
+    "allreduce_quantized",
+    "get_padded_sizes",
+    "reduce_scatter_quantized",
     "fused_dequantize_from_fp8",
     "fused_quantize_into_fp8",
     "fused_reduce_fp8",
