@@ -43,7 +43,11 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--sets", type=int, default=3, help="buffer sets the steps rotate over")
-    ap.add_argument("--rank", type=int, default=3)
+    ap.add_argument("--rank", type=int, default=None)
+    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat"],
+                    help="workload: 3 = Llama-3-8B layer bucket (the headline, default); 2, 4, 5 = the "
+                         "other GPU configurations; flat = one 1-D fp32 tensor of 64 Mi elements "
+                         "(what a bucketised DiLoCo all-reduce passes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a counter "
@@ -128,8 +132,27 @@ def main() -> int:
         print("bench.py: " + _lib.strerror(rc), file=sys.stderr)
         return 2
 
-    ws, rank, op = 8, args.rank, ReduceOp.AVG
     dev = "cuda"
+    cfg5_shapes = workloads.cfg5_shapes(10000) if args.config == "5" else None
+    table = {
+        "2": (lambda seed: workloads.cfg2(seed, device=dev), 8, ReduceOp.AVG,
+              "config 2: one bf16 tensor [4096, 4096], N(0, 0.02), ws=8, AVG"),
+        "3": (lambda seed: workloads.cfg3(seed, device=dev), 8, ReduceOp.AVG,
+              "BASELINE config 3: Llama-3-8B decoder-layer gradient bucket, "
+              "9 bf16 tensors, 218112000 elements, ws=8, reduce AVG"),
+        "4": (lambda seed: workloads.cfg4(seed, device=dev), 4, ReduceOp.AVG,
+              "config 4: DiLoCo pseudo-gradient of a 1.1B model, 201 fp32 tensors, "
+              "1100048384 elements, Student-t(3) x 1e-4, ws=4, AVG"),
+        "5": (lambda seed: workloads.cfg5(seed, torch.bfloat16, cfg5_shapes, device=dev), 16,
+              ReduceOp.SUM, "config 5: 10000 bf16 tensors of 1..4096 elements, ragged rows, ws=16, SUM"),
+        "flat": (lambda seed: [torch.randn(64 * 1024 * 1024, device=dev,
+                                           generator=torch.Generator(device=dev).manual_seed(seed))],
+                 8, ReduceOp.SUM, "one 1-D fp32 tensor of 67108864 elements (rows of one column), ws=8, SUM"),
+    }
+    make, ws, op, workload_name = table[args.config]
+    rank = args.rank if args.rank is not None else min(3, ws - 1)
+    if args.config == "4":
+        args.sets = min(args.sets, 2)
 
     # ---- buffer sets: tensors, received buffer B, gathered buffer G ----------
     sets = []
@@ -137,7 +160,7 @@ def main() -> int:
         slots = []
         mine = None
         for peer in range(ws):
-            t = workloads.cfg3(1000 * k + peer, device=dev)
+            t = make(1000 * k + peer)
             qp = q.fused_quantize_into_fp8(t, ws)
             slot = qp.numel() // ws
             slots.append(qp[rank * slot:(rank + 1) * slot].clone())
@@ -153,7 +176,9 @@ def main() -> int:
 
     # ---- parity gate on the data that is being timed -------------------------
     from oracle import oracle
-    probe = [sets[0]["tensors"][1]]  # k_proj gradient [1024, 4096]
+    # a mid-sized tensor of the first set (config 3: the k_proj gradient [1024, 4096])
+    cand = sets[0]["tensors"]
+    probe = [cand[1] if len(cand) > 1 else cand[0][: min(cand[0].shape[0], 2048)]]
     probe_cpu = [probe[0].cpu()]
     qg = q.fused_quantize_into_fp8(probe, ws)
     qc = oracle.fused_quantize_into_fp8(list(probe_cpu), ws)
@@ -165,7 +190,7 @@ def main() -> int:
     dg, dc = [torch.empty_like(probe[0])], [torch.empty_like(probe_cpu[0])]
     q.fused_dequantize_from_fp8(dg, qg, ws)
     oracle.fused_dequantize_from_fp8(dc, qc, ws)
-    ok = ok and torch.equal(dg[0].cpu().view(torch.int16), dc[0].view(torch.int16))
+    ok = ok and torch.equal(dg[0].cpu().reshape(-1).view(torch.uint8), dc[0].reshape(-1).view(torch.uint8))
     if not ok:
         print("bench.py: GPU results differ from the CPU checker", file=sys.stderr)
         return 1
@@ -239,21 +264,21 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "BASELINE config 3: Llama-3-8B decoder-layer gradient bucket, "
-                               "9 bf16 tensors, 218112000 elements, ws=8, reduce AVG, rank "
-                               f"{rank}; {len(sets)} rotating buffer sets (cold last-level cache)",
-                   "input_dtype": "bf16", "packed_bytes": int(sets[0]["gathered"].numel()),
+        "config": {"workload": f"{workload_name}, rank {rank}; {len(sets)} rotating buffer sets "
+                               "(cold last-level cache)",
+                   "input_dtype": str(sets[0]["tensors"][0].dtype).replace("torch.", ""),
+                   "packed_bytes": int(sets[0]["gathered"].numel()),
                    "algorithmic_bytes_per_step": total_bytes},
-        "roofline": {"bound": "hbm", "kernel": "k_quantize<bf16>",
+        "roofline": {"bound": "hbm", "kernel": "k_quantize",
                      "achieved": stages["quantize"]["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": stages["quantize"]["frac"],
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated
                      # on a 256 MiB copy) + WRITE_SIZE (x1.000); profiles/cfg3_bf16_ws8_hbm_traffic.md
-                     "traffic": 654846000},
+                     "traffic": 654846000 if args.config == "3" else None},
         "stages": stages,
         "parity": "quantize, reduce, dequantize byte-identical to the CPU checker on the probe tensor",
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.config == "3":
         out["cpu_baseline"] = cpu_baseline(args.cpu_rows)
     print(json.dumps(out))
     return 0

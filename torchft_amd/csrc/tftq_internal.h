@@ -21,6 +21,7 @@ enum : uint8_t {
     K_GEN8 = 5,    // 8 lanes per row
     K_GEN64 = 6,   // one wavefront per row
     K_GEN256 = 7,  // one workgroup per row (reduce only)
+    K_COL1 = 8,    // rows of a single column (1-D tensors): 4 rows per lane, 1024 per workgroup
 };
 
 static inline int tftq_team_of(uint8_t kind)

@@ -409,6 +409,35 @@ DEV void quantize_gen(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
+// Rows of one column (1-D tensors, quantization.py:487-488): a row is its own
+// maximum, so the code is +-448 (or 0) and all information is in the scale.
+// Four rows per lane, interleaved so that every load and every 8-byte
+// [scale, code] store of a wavefront is contiguous.
+template <typename T>
+DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+{
+    const int m_pad = s.slice_rows * p.ws;
+    float x[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = min(row0 + k * TFTQ_WG + tid, s.m - 1);
+        x[k] = s.m > 0 ? Elem<T>::load(s.ptr, (int64_t)row * s.row_stride) : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = row0 + k * TFTQ_WG + tid;
+        if (row < m_pad) {
+            u32x2 o = {0u, 0u};  // padding rows stay zero
+            if (row < s.m) {
+                const float sc = calc_scale(__builtin_fabsf(x[k]));
+                o.x = as_u(sc);
+                o.y = pack_fp8x4(x[k] * sc, 0.0f, 0.0f, 0.0f) & 0xFFu;
+            }
+            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + row_addr(s, p.slot_size, row)) = o;
+        }
+    }
+}
+
 template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
@@ -429,6 +458,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
         break;
     case K_GEN8: quantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: quantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
+    case K_COL1: quantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid); break;
     default: break;
     }
 }
@@ -507,6 +537,24 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
+// Rows of one column: one plain divide per row, four rows per lane.
+template <typename T>
+DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+{
+    u32x2 w[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = min(row0 + k * TFTQ_WG + tid, s.m - 1);
+        w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)as_global<const u32>(p.packed + row_addr(s, p.slot_size, row)));
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = row0 + k * TFTQ_WG + tid;
+        const float f = __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0);
+        if (row < s.m) Elem<T>::store(s.ptr, (int64_t)row * s.row_stride, f / as_f(w[k].x));  // no zero guard (:239)
+    }
+}
+
 template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const InlineTable inl)
 {
@@ -526,6 +574,9 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
         break;
     case K_GEN8: dequantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: dequantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
+    case K_COL1:
+        if (s.m > 0) dequantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid);
+        break;
     default: break;
     }
 }
@@ -892,6 +943,40 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
     }
 }
 
+// Rows of one column: 8 bytes per row and peer, one plain divide per peer
+// (coefficients for the fast division would cost two), four rows per lane.
+template <bool GDIV>
+DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
+{
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    int64_t off[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        off[k] = s.slot_off + (int64_t)min(j0 + k * TFTQ_WG + tid, s.slice_rows - 1) * 8;
+#pragma nounroll
+    for (int kk = 0; kk < p.ws; kk++) {
+        u32x2 w[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)peer_row(p, kk, off[k]));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float sc = as_f(w[k].x);
+            sc = sc == 0.0f ? 1.0f : sc;  // padding rows (:419)
+            acc[k] = acc[k] + __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0) / sc;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        if (j0 + k * TFTQ_WG + tid < s.slice_rows) {
+            const float s2 = calc_scale(__builtin_fabsf(acc[k]) / p.div);
+            u32x2 o;
+            o.x = as_u(s2);
+            o.y = pack_fp8x4(scale_div<GDIV>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
+            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off[k]) = o;
+        }
+    }
+}
+
 template <bool INLINE, bool GDIV>
 __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
 {
@@ -916,6 +1001,8 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
             }
         } else if (ndw <= 1024) {
             reduce_rows<256, 1, true, GDIV>(s, p, j0, nrows, tid, lds);
+        } else if (ndw <= 2048) {
+            reduce_rows<256, 2, true, GDIV>(s, p, j0, nrows, tid, lds);
         } else {
             reduce_rows<256, 4, false, GDIV>(s, p, j0, nrows, tid, lds);
         }
@@ -925,14 +1012,20 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         const int j0 = (blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6)) * rpt;
         const int nrows = min(rpt, s.slice_rows - j0);
         if (p.ws > 64 || (ndw & 3) != 0) {
-            for (int r = 0; r < nrows; r++) reduce_row<64, 1, GDIV>(s, p, j0 + r, tid & 63, lds);
-        } else {
+            for (int r = 0; r < nrows; r++) {
+                if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j0 + r, tid & 63, lds);
+                else reduce_row<64, 2, GDIV>(s, p, j0 + r, tid & 63, lds);
+            }
+        } else if (ndw <= 256) {
             reduce_rows<64, 1, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
+        } else {
+            reduce_rows<64, 2, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
         }
         break;
     }
     case K_GEN8: reduce_row<8, 1, GDIV>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
     case K_GEN1: reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds); break;
+    case K_COL1: reduce_col1<GDIV>(s, p, blk * 4 * TFTQ_WG, tid); break;
     default: break;
     }
 }

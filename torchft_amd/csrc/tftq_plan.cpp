@@ -58,6 +58,7 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     const bool vec_ok = s.ptr != 0 && s.n > 0 && s.n % epv == 0 && s.col_stride == 1 &&
                         s.ptr % 16 == 0 && (s.m <= 1 || (s.row_stride * esz) % 16 == 0) &&
                         in_bytes >= 64;
+    if (s.n == 1 && s.ptr != 0) return K_COL1;
     if (vec_ok) {
         if (in_bytes <= 1024) return K_VEC8;
         if (in_bytes <= 8192) return K_VEC64;
@@ -70,11 +71,12 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
 
 static uint8_t pick_reduce_kind(const Seg &s)
 {
-    // one 16-byte vector of codes per lane and peer, except for the longest rows
+    // one or two 16-byte vectors of codes per lane and peer, four for the longest rows
     const int ndw = s.row_bytes / 4 - 1;
+    if (s.n == 1) return K_COL1;
     if (ndw <= 4) return K_GEN1;
     if (ndw <= 32) return K_GEN8;
-    if (ndw <= 256) return K_GEN64;
+    if (ndw <= 512) return K_GEN64;
     return K_GEN256;
 }
 
@@ -95,6 +97,7 @@ static int pick_reduce_rows(const Seg &s, int ws)
 
 static int rows_per_wg_of(const Seg &s, int st)
 {
+    if (s.kind[st] == K_COL1) return 4 * TFTQ_WG;
     const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
     return st == ST_R ? teams * s.reduce_rows_per_team : teams;
 }
