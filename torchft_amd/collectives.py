@@ -163,12 +163,13 @@ def reduce_scatter_quantized(
     ]
 
     with cuda.stream(ex.stream):
-        packed = _q.fused_quantize_into_fp8(inputs, ws)
+        plan, device = _q._prepare(inputs, ws)  # one walk over the list for both kernels
+        packed = _q._quantize(plan, device)
         received, work = ex.scatter_slots(packed)
         work.wait()
 
         def reduce_then_dequantize() -> None:
-            _q.fused_reduce_fp8(inputs, received, ws, rank, ex.reduce_op)
+            _q._reduce(plan, device, received, rank, ex.reduce_op)
             own = received.view(ws, -1).split(1)[rank].squeeze(0)
             # one slot has the layout of a group of one over the [m_pad / ws, n] shares
             _q.fused_dequantize_from_fp8(share_views, own, 1)
@@ -193,12 +194,13 @@ def allreduce_quantized(
     ws, rank = ex.world_size, ex.rank
 
     with cuda.stream(ex.stream):
-        packed = _q.fused_quantize_into_fp8(tensors, ws)
+        plan, device = _q._prepare(tensors, ws)  # one walk over the list for all three kernels
+        packed = _q._quantize(plan, device)
         received, a2a = ex.scatter_slots(packed)
         a2a.wait()
-        _q.fused_reduce_fp8(tensors, received, ws, rank, ex.reduce_op)
+        _q._reduce(plan, device, received, rank, ex.reduce_op)
         # the reduced slots of all ranks land in the first buffer
         work = ex.gather_slots(packed, received)
         work.wait()  # a stream dependency with RCCL, not a host block
-        ex.finish_on_stream(work, lambda: _q.fused_dequantize_from_fp8(tensors, packed, ws))
+        ex.finish_on_stream(work, lambda: _q._dequantize(plan, device, packed))
     return work

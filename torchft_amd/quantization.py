@@ -142,6 +142,37 @@ def _check_packed(output: torch.Tensor, plan: _Plan) -> None:
         raise RuntimeError("the packed buffer must be a contiguous uint8 tensor")
 
 
+# The three stages on a prepared plan.  The public functions below prepare and
+# call these; torchft_amd.collectives prepares once per collective and calls
+# all three, which saves two walks over the tensor list.
+def _quantize(plan: _Plan, device: torch.device) -> torch.Tensor:
+    with torch.cuda.device(device):
+        # float32 storage like the reference (:567-571) so that scales are aligned
+        output = torch.empty(plan.output_size // SCALE_DTYPE_BYTES, device=device,
+                             dtype=SCALE_DTYPE).view(torch.uint8)
+        _check(plan._lib.tftq_quantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                       plan.output_size, _stream_ptr(device)), "tftq_quantize")
+    return output
+
+
+def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
+            reduce_op: ReduceOp) -> None:
+    _check_packed(output, plan)
+    is_avg = 0 if reduce_op == ReduceOp.SUM else 1  # anything but SUM averages (:682)
+    with torch.cuda.device(device):
+        _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                     plan.output_size, int(rank), is_avg,
+                                     _stream_ptr(device)), "tftq_reduce")
+
+
+def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor) -> None:
+    _check_packed(output, plan)
+    with torch.cuda.device(device):
+        _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                         plan.output_size, _stream_ptr(device)),
+               "tftq_dequantize")
+
+
 def fused_quantize_into_fp8(
     inputs: list[torch.Tensor], all_reduce_group_size: int
 ) -> torch.Tensor:
@@ -158,13 +189,7 @@ def fused_quantize_into_fp8(
         the packed uint8 tensor (``numel() % all_reduce_group_size == 0``)
     """
     plan, device = _prepare(inputs, all_reduce_group_size)
-    with torch.cuda.device(device):
-        # float32 storage like the reference (:567-571) so that scales are aligned
-        output = torch.empty(plan.output_size // SCALE_DTYPE_BYTES, device=device,
-                             dtype=SCALE_DTYPE).view(torch.uint8)
-        _check(plan._lib.tftq_quantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                       plan.output_size, _stream_ptr(device)), "tftq_quantize")
-    return output
+    return _quantize(plan, device)
 
 
 def fused_dequantize_from_fp8(
@@ -176,11 +201,7 @@ def fused_dequantize_from_fp8(
     quantized.
     """
     plan, device = _prepare(inputs, all_reduce_group_size)
-    _check_packed(output, plan)
-    with torch.cuda.device(device):
-        _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                         plan.output_size, _stream_ptr(device)),
-               "tftq_dequantize")
+    _dequantize(plan, device, output)
 
 
 def fused_reduce_fp8(
@@ -197,9 +218,4 @@ def fused_reduce_fp8(
     ``inputs`` only supplies the shapes.
     """
     plan, device = _prepare(inputs, all_reduce_group_size)
-    _check_packed(output, plan)
-    is_avg = 0 if reduce_op == ReduceOp.SUM else 1
-    with torch.cuda.device(device):
-        _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                     plan.output_size, int(all_reduce_rank), is_avg,
-                                     _stream_ptr(device)), "tftq_reduce")
+    _reduce(plan, device, output, all_reduce_rank, reduce_op)
