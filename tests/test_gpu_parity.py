@@ -303,6 +303,81 @@ def test_cfg3_full_size(q, oracle):
         assert torch.equal(a, b)
 
 
+def test_cfg4_full_size(q, oracle):
+    """The whole 1.1 B-parameter fp32 pseudo-gradient (201 tensors, 4.4 GB per peer,
+    ws = 4, AVG), generated on the GPU.  Three tensors of different row classes are
+    checked byte for byte against the checker inside the full packed buffers; the
+    rest through properties that do not depend on size."""
+    ws, rank = 4, 2
+    mine = workloads.cfg4(rank, device="cuda")
+    assert len(mine) == 201 and sum(t.numel() for t in mine) == 1100048384
+    packed = q.fused_quantize_into_fp8(mine, ws)
+    assert packed.numel() == 1102526464
+    shapes = [tuple(t.shape) for t in mine]
+    offs, slot, total = oracle.layout(shapes, ws)
+    picks = [3, 7, 9, 199]  # v_proj [256, 2048], down_proj [2048, 5632], a norm [2048, 1], final norm
+    for i in picks:
+        m, n = shapes[i]
+        want = oracle.fused_quantize_into_fp8([mine[i].cpu()], ws, nthreads=NT)
+        sr, rb = -(-m // ws), (-(-n // 4) + 1) * 4
+        for p in range(ws):
+            got = packed[p * slot + offs[i]: p * slot + offs[i] + sr * rb].cpu()
+            assert torch.equal(got, want[p * sr * rb:(p + 1) * sr * rb]), (i, p)
+    # every scale is 448 / amax (or 1.0), every row's arg-max encodes to +-448
+    for i in (0, 5, 200):
+        x = mine[i]
+        m, n = x.shape
+        sr, rb = -(-m // ws), (-(-n // 4) + 1) * 4
+        rows = torch.cat([packed[p * slot + offs[i]: p * slot + offs[i] + sr * rb].view(sr, rb)
+                          for p in range(ws)])[:m]
+        scales = rows[:, :4].contiguous().view(torch.float32).view(m)
+        amax = x.abs().amax(dim=1)
+        want_s = torch.where(amax > 0, torch.tensor(448.0, device="cuda") / amax, torch.ones_like(amax))
+        assert torch.equal(scales, want_s)
+        top = rows[torch.arange(m, device="cuda"), 4 + x.abs().argmax(dim=1)] & 0x7F
+        assert ((top == 0x7E) | (amax == 0)).all()
+    # reduce of 4 identical peers with AVG gives back the same codes (-0 becomes +0); scales
+    # within 4 fp32 ulps
+    recv = packed[rank * slot:(rank + 1) * slot].repeat(ws)
+    before = recv[rank * slot:(rank + 1) * slot].clone()
+    q.fused_reduce_fp8(mine, recv, ws, rank, ReduceOp.AVG)
+    after = recv[rank * slot:(rank + 1) * slot]
+    for i in (0, 7, 200):
+        m, n = shapes[i]
+        sr, rb = -(-m // ws), (-(-n // 4) + 1) * 4
+        a = after[offs[i]: offs[i] + sr * rb].view(sr, rb)
+        b = before[offs[i]: offs[i] + sr * rb].view(sr, rb)
+        real = min(sr, max(0, m - rank * sr))
+        want = b[:real, 4:].clone()
+        want[want == 0x80] = 0  # a sum of negative zeros is +0
+        assert torch.equal(a[:real, 4:], want)
+        da = a[:real, :4].contiguous().view(torch.int32) - b[:real, :4].contiguous().view(torch.int32)
+        assert da.abs().max() <= 4
+    del recv, before
+    # round trip: dequantize(quantize(x)) is within half an fp8 ULP of x, row by row
+    outs = [torch.empty_like(t) for t in mine]
+    q.fused_dequantize_from_fp8(outs, packed, ws)
+    for x, o in zip(mine, outs):
+        amax = x.abs().amax(dim=1, keepdim=True)
+        tol = torch.maximum(x.abs() * 2 ** -4, amax * (2 ** -10 / 448.0)) * 1.001
+        assert ((x - o).abs() <= tol).all()
+
+
+def test_cfg5_full_size(q, oracle):
+    """All 10 000 ragged tensors, 16 peers, SUM: every peer's packed buffer, three
+    ranks' reductions and the dequantized result against the checker."""
+    shapes = workloads.cfg5_shapes(10000)
+    peers = [workloads.cfg5(s, torch.bfloat16, shapes) for s in range(16)]
+    full_check(q, oracle, peers, 16, ReduceOp.SUM, ranks=[0, 9, 15])
+    outs_g = [torch.empty_like(t).cuda() for t in peers[3]]
+    outs_c = [torch.empty_like(t) for t in peers[3]]
+    buf = oracle.fused_quantize_into_fp8(list(peers[3]), 16, nthreads=NT)
+    q.fused_dequantize_from_fp8(outs_g, buf.cuda(), 16)
+    oracle.fused_dequantize_from_fp8(outs_c, buf, 16, nthreads=NT)
+    for a, b in zip(outs_g, outs_c):
+        assert torch.equal(a.cpu().view(-1).view(torch.uint8), b.view(-1).view(torch.uint8))
+
+
 # ---- memory safety around the packed buffer ---------------------------------------
 def test_no_write_outside_packed_buffer(q):
     """Calls the C ABI with a packed buffer placed between two canary zones."""
