@@ -215,6 +215,40 @@ def test_strided_and_misaligned_inputs(q, oracle, dtype):
     same_bytes(gof, of, "strided dequantize flat")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_unaligned_rows_and_tails(q, oracle, dtype):
+    """Contiguous rows whose start or length is not a multiple of 16 bytes take the
+    vector kinds with element-aligned 16-byte accesses and a per-element tail."""
+    g = torch.Generator().manual_seed(17)
+    esz = 4 if dtype == torch.float32 else 2
+    cases = []
+    for n in (33, 67, 130, 515, 1023, 4092, 4099, 9001):
+        flat = torch.randn(6 * n + 7, generator=g).to(dtype)
+        for off in (0, 1, 3):
+            cases.append((flat, off, 5, n))
+    cpu_views = [f[o:o + m * n].view(m, n) for f, o, m, n in cases]
+    gpu_flats = {id(f): f.cuda() for f, _, _, _ in cases}
+    gpu_views = [gpu_flats[id(f)][o:o + m * n].view(m, n) for f, o, m, n in cases]
+    assert any(v.data_ptr() % 16 != 0 for v in gpu_views)
+    for ws in (1, 4):
+        a = q.fused_quantize_into_fp8(list(gpu_views), ws)
+        b = oracle.fused_quantize_into_fp8(list(cpu_views), ws)
+        same_bytes(a, b, f"unaligned quantize ws={ws}")
+        red_g, red_c = a.clone(), b.clone()
+        q.fused_reduce_fp8(list(gpu_views), red_g, ws, ws - 1, ReduceOp.AVG)
+        oracle.fused_reduce_fp8(list(cpu_views), red_c, ws, ws - 1, ReduceOp.AVG)
+        same_bytes(red_g, red_c, f"unaligned reduce ws={ws}")
+        # dequantize into fresh unaligned destinations (distinct storage per case)
+        out_c = [torch.full((m * n + 8,), 5.0, dtype=dtype) for _, _, m, n in cases]
+        out_g = [t.cuda() for t in out_c]
+        dst_c = [t[o:o + m * n].view(m, n) for t, (_, o, m, n) in zip(out_c, cases)]
+        dst_g = [t[o:o + m * n].view(m, n) for t, (_, o, m, n) in zip(out_g, cases)]
+        oracle.fused_dequantize_from_fp8(list(dst_c), b, ws)
+        q.fused_dequantize_from_fp8(list(dst_g), a, ws)
+        for i, (x, y) in enumerate(zip(out_g, out_c)):
+            same_bytes(x, y, f"unaligned dequantize case {i} ws={ws}")  # guard elements included
+
+
 @pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (3, ReduceOp.AVG), (5, ReduceOp.SUM),
                                    (6, ReduceOp.AVG), (70, ReduceOp.AVG), (64, ReduceOp.SUM)])
 def test_group_sizes(q, oracle, ws, op):

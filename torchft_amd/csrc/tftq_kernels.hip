@@ -39,6 +39,7 @@ typedef u32 u32x4 __attribute__((ext_vector_type(4)));
 typedef u32 u32x2 __attribute__((ext_vector_type(2)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x2 u32x2_a4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));  // tensor rows: aligned to the element only
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -348,13 +349,24 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
 
     constexpr int EPV = Elem<T>::EPV;
     const int nvec = s.n / EPV;
-    GLOBAL const u32x4 *in = as_global<const u32x4>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
+    const int tail = s.n - nvec * EPV;  // elements after the last whole vector (rare)
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
     u32x4 v[KMAX];
 #pragma unroll
     for (int k = 0; k < KMAX; k++) v[k] = LOAD_STREAM(in + min(k * TEAM + lane, nvec - 1));
+    float t[EPV - 1];
+    if (tail) {  // every lane reads the few tail elements; lane 0 will store their codes
+#pragma unroll
+        for (int e = 0; e < EPV - 1; e++) t[e] = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(e, tail - 1));
+    }
     float amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < KMAX; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+    if (tail) {
+#pragma unroll
+        for (int e = 0; e < EPV - 1; e++) amax = fmaxf(amax, __builtin_fabsf(t[e]));
+    }
     amax = team_max<TEAM>(amax, lds);
     const float sc = calc_scale(amax);
     if (lane == 0) out[0] = as_u(sc);
@@ -362,6 +374,20 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     for (int k = 0; k < KMAX; k++) {
         const int idx = k * TEAM + lane;
         if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
+    }
+    if (tail && lane == 0) {
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) y[e] = (e < EPV - 1 && e < tail) ? t[e < EPV - 1 ? e : 0] * sc : 0.0f;
+        GLOBAL u32 *tw = out + 1 + nvec * (EPV / 4);
+        u32 w0 = pack_fp8x4(y[0], y[1], y[2], y[3]);
+        if (tail < 4) w0 &= (1u << (8 * tail)) - 1u;  // padding bytes are zero whatever 0 * sc gave
+        tw[0] = w0;
+        if (EPV == 8 && tail > 4) {
+            u32 w1 = pack_fp8x4(y[4], y[5], y[6], y[7]);
+            if (tail < 8) w1 &= (1u << (8 * (tail - 4))) - 1u;
+            tw[1] = w1;
+        }
     }
 }
 
@@ -506,7 +532,12 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
     constexpr int EPV = Elem<T>::EPV;
     constexpr int DV = 4;
     const int nvec = s.n / EPV;
-    GLOBAL u32x4 *out = as_global<u32x4>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
+    GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
+    // the few columns after the last whole vector, one element per lane
+    for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
+        const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
+        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, div_fast_signed(f, c.r, c.r_lo));
+    }
     for (int base = 0; base < nvec; base += DV * TEAM) {
         u32x2 w[DV];
 #pragma unroll
@@ -819,7 +850,7 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 // no branch: a lane past the end of the row re-reads the row's last vector, a
 // batch past the last peer re-reads the last peer, and both are ignored later.
 // Needs TEAM >= 64 (a peer's scale lives in one lane of each wavefront),
-// ws <= 64 and rows that are a whole number (>= 1) of 16-byte vectors.
+// ws <= 64 and rows of at least one 16-byte vector.
 constexpr int R_VPB = 4;
 
 template <int TEAM, int UNITS, bool PIPE, bool GDIV>
@@ -827,16 +858,24 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
 {
     constexpr int PB = R_VPB / UNITS >= 1 ? R_VPB / UNITS : 1;  // peers per batch
     if (nrows <= 0) return;
-    const int nvec = ((s.row_bytes >> 2) - 1) >> 2;
+    const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
     const int ws = p.ws;
     const int nb = (ws + PB - 1) / PB;  // batches per row
     const int total = nrows * nb;
     const int wlane = threadIdx.x & 63;
     const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
 
-    int vidx[UNITS];
+    // Vector u of this lane starts at dword doff[u].  The last vector of a row whose
+    // length is not a multiple of 4 dwords is moved back so that it ends with the row:
+    // it overlaps its neighbour, both lanes compute and store the same values.  Lanes
+    // past the row's end re-read the last vector and do not store.
+    int doff[UNITS];
+    u32 padmask[UNITS];  // clears the bytes past column n in the row's last dword (:420-424)
 #pragma unroll
-    for (int u = 0; u < UNITS; u++) vidx[u] = min(u * TEAM + lane, nvec - 1);
+    for (int u = 0; u < UNITS; u++) {
+        doff[u] = min(4 * (u * TEAM + lane), ndw - 4);
+        padmask[u] = (doff[u] == ndw - 4 && (s.n & 3)) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+    }
 
     struct Batch {
         u32x4 w[PB][UNITS];
@@ -850,10 +889,12 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
         dst.scale = as_f(peer_row(p, speer, off)[0]);
 #pragma unroll
         for (int b = 0; b < PB; b++) {
-            GLOBAL const u32x4_a4 *pv =
-                (GLOBAL const u32x4_a4 *)(peer_row(p, min(lbatch * PB + b, ws - 1), off) + 1);
+            GLOBAL const u32 *pv = peer_row(p, min(lbatch * PB + b, ws - 1), off) + 1;
 #pragma unroll
-            for (int u = 0; u < UNITS; u++) dst.w[b][u] = LOAD_STREAM(pv + vidx[u]);
+            for (int u = 0; u < UNITS; u++) {
+                dst.w[b][u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + doff[u]));
+                dst.w[b][u].w &= padmask[u];
+            }
         }
         if (++lbatch == nb) {
             lbatch = 0;
@@ -904,7 +945,7 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
 #pragma unroll
                 for (int u = 0; u < UNITS; u++) {
                     const u32x4 o = requant16<GDIV>(acc[u], s2, p);
-                    if (u * TEAM + lane < nvec) ((GLOBAL u32x4_a4 *)(orow + 1))[u * TEAM + lane] = o;
+                    if (4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
                 }
                 if (lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
             } else {
@@ -994,7 +1035,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         const int nrows = min(rpt, s.slice_rows - j0);
         if (ndw > 4096) {
             for (int r = 0; r < nrows; r++) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
-        } else if (p.ws > 64 || (ndw & 3) != 0) {
+        } else if (p.ws > 64) {
             for (int r = 0; r < nrows; r++) {
                 if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j0 + r, tid, lds);
                 else reduce_row<256, 4, GDIV>(s, p, j0 + r, tid, lds);
@@ -1011,7 +1052,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
     case K_GEN64: {
         const int j0 = (blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6)) * rpt;
         const int nrows = min(rpt, s.slice_rows - j0);
-        if (p.ws > 64 || (ndw & 3) != 0) {
+        if (p.ws > 64) {
             for (int r = 0; r < nrows; r++) {
                 if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j0 + r, tid & 63, lds);
                 else reduce_row<64, 2, GDIV>(s, p, j0 + r, tid & 63, lds);

@@ -53,11 +53,11 @@ extern "C" int tftq_layout(int n_tensors, const int64_t *shapes, int ws, int64_t
 
 static uint8_t pick_io_kind(const Seg &s, int esz)
 {
-    const int epv = 16 / esz;
+    // Vector kinds: contiguous rows of at least 64 bytes.  Neither the row start nor the
+    // row length needs to be a multiple of 16 bytes: gfx950 loads and stores 16-byte
+    // vectors at element alignment, and a short tail is handled per element.
     const int64_t in_bytes = (int64_t)s.n * esz;
-    const bool vec_ok = s.ptr != 0 && s.n > 0 && s.n % epv == 0 && s.col_stride == 1 &&
-                        s.ptr % 16 == 0 && (s.m <= 1 || (s.row_stride * esz) % 16 == 0) &&
-                        in_bytes >= 64;
+    const bool vec_ok = s.ptr != 0 && s.col_stride == 1 && in_bytes >= 64;
     if (s.n == 1 && s.ptr != 0) return K_COL1;
     if (vec_ok) {
         if (in_bytes <= 1024) return K_VEC8;
