@@ -265,8 +265,11 @@ def test_long_rows(q, oracle):
     g = torch.Generator().manual_seed(21)
     for dtype in (torch.bfloat16, torch.float32):
         peers = [[(torch.randn(5, 20000, generator=g)).to(dtype),
-                  (torch.randn(3, 70000, generator=g)).to(dtype)] for _ in range(2)]
+                  (torch.randn(3, 70000, generator=g)).to(dtype),
+                  (torch.randn(4, 70003, generator=g)).to(dtype),
+                  (torch.randn(40001 * 2 + 1, generator=g)).to(dtype)[1:].view(2, 40001)] for _ in range(2)]
         full_check(q, oracle, peers, 2, ReduceOp.AVG)
+        full_check(q, oracle, peers * 2, 4, ReduceOp.SUM, ranks=[3])
 
 
 def test_extreme_scales_and_denormals(q, oracle):

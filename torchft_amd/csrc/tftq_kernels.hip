@@ -391,12 +391,64 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     }
 }
 
+// Rows of more than 32 KB: too long for the registers of a workgroup.  Two
+// passes with 16-byte loads; the second one finds the row in the caches.
+template <typename T>
+DEV void quantize_vec_long(const Seg &s, const KParams &p, int row, int tid, float *lds)
+{
+    const bool active = row < s.slice_rows * p.ws;
+    if (!active) return;
+    GLOBAL u32 *out = as_global<u32>(p.packed + row_addr(s, p.slot_size, row));
+    if (row >= s.m) {
+        for (int d = tid; d < (s.row_bytes >> 2); d += TFTQ_WG) out[d] = 0;
+        return;
+    }
+    constexpr int EPV = Elem<T>::EPV;
+    const int nvec = s.n / EPV;
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
+    float amax = 0.0f;
+    for (int c = nvec * EPV + tid; c < s.n; c += TFTQ_WG) amax = fmaxf(amax, __builtin_fabsf(Elem<T>::load(s.ptr, r0 + c)));
+#pragma nounroll
+    for (int base = 0; base < nvec; base += 4 * TFTQ_WG) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = in[min(base + k * TFTQ_WG + tid, nvec - 1)];
+#pragma unroll
+        for (int k = 0; k < 4; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+    }
+    amax = team_max<256>(amax, lds);
+    const float sc = calc_scale(amax);
+    if (tid == 0) out[0] = as_u(sc);
+#pragma nounroll
+    for (int base = 0; base < nvec; base += 4 * TFTQ_WG) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = LOAD_STREAM(in + min(base + k * TFTQ_WG + tid, nvec - 1));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int idx = base + k * TFTQ_WG + tid;
+            if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
+        }
+    }
+    // tail: at most EPV - 1 elements after the last whole vector, byte stores plus zero padding
+    if (tid == 0) {
+        const int c0 = nvec * EPV;
+        GLOBAL uint8_t *ob = (GLOBAL uint8_t *)(out + 1);
+        for (int c = c0; c < ((s.n + 3) & ~3); c++) {
+            const float x = c < s.n ? Elem<T>::load(s.ptr, r0 + c) : 0.0f;
+            ob[c] = c < s.n ? (uint8_t)(pack_fp8x4(x * sc, 0.0f, 0.0f, 0.0f) & 0xFFu) : (uint8_t)0;
+        }
+    }
+}
+
 template <typename T, int TEAM>
 DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds)
 {
     // same branch for the whole workgroup
     if (s.n / Elem<T>::EPV <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
-    else quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
+    else if (TEAM < 256 || s.n / Elem<T>::EPV <= QV * TEAM) quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
+    else quantize_vec_long<T>(s, p, row, lane, lds);
 }
 
 // Any strides, any alignment, any n: element loads, two passes over the row
@@ -743,6 +795,65 @@ DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float 
     if (lane == 0) *(GLOBAL u32 *)orow = as_u(s2);
 }
 
+// Rows longer than a 256-lane team can keep in registers (more than 16384
+// columns): two passes over chunks of 1024 dwords, as the reference does for
+// every row (:318-372), but with 16-byte loads, the fast exact division and the
+// scales read once.  The second pass finds the peer rows in the caches.
+template <bool GDIV>
+DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *lds)
+{
+    const int ndw = (s.row_bytes >> 2) - 1;
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    const int wlane = tid & 63;
+    const int ws = p.ws;  // <= 64 here
+    const DivCoef c = make_div(guarded_scale(peer_row(p, min(wlane, ws - 1), off)));
+    if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // same in the four wavefronts
+        reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
+        return;
+    }
+    GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+    const u32 tailmask = (s.n & 3) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+    float amax = 0.0f, s2 = 0.0f;
+#pragma nounroll
+    for (int pass = 0; pass < 2; pass++) {
+#pragma nounroll
+        for (int d = 0; d < ndw; d += 4 * TFTQ_WG) {
+            const bool valid = d + 4 * tid < ndw;
+            const int doff = min(d + 4 * tid, ndw - 4);  // the last vector ends with the row
+            const u32 mask = doff == ndw - 4 ? tailmask : 0xFFFFFFFFu;
+            float acc[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+#pragma nounroll
+            for (int k0 = 0; k0 < ws; k0 += 4) {
+                u32x4 w[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k0 + b, ws - 1), off) + 1 + doff));
+                    w[b].w &= mask;
+                }
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+                    if (k0 + b < ws) accumulate16(acc, w[b], bcast_lane(c.r, k0 + b), bcast_lane(c.r_lo, k0 + b));
+            }
+            if (pass == 0) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[e]));
+            } else {
+                // the moved-back last vector overlaps its neighbour, which may sit in another
+                // wavefront: nobody stores before everybody has read the own slot's chunk
+                __syncthreads();
+                if (valid) *(GLOBAL u32x4_a4 *)(orow + 1 + doff) = requant16<GDIV>(acc, s2, p);
+            }
+        }
+        if (pass == 0) {
+            amax = team_max<256>(amax, lds);  // every wavefront has read the old scales by now
+            s2 = calc_scale(amax / p.div);
+        }
+    }
+    if (tid == 0) orow[0] = as_u(s2);  // :375
+}
+
 // Register-resident row: the team holds all accumulators of the row, each peer
 // row is read once.  UNITS = 16-byte vectors of codes per lane and peer.
 template <int TEAM, int UNITS, bool GDIV>
@@ -1034,7 +1145,10 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         const int j0 = blk * rpt;
         const int nrows = min(rpt, s.slice_rows - j0);
         if (ndw > 4096) {
-            for (int r = 0; r < nrows; r++) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
+            for (int r = 0; r < nrows; r++) {
+                if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
+                else reduce_row_long<GDIV>(s, p, j0 + r, tid, lds);
+            }
         } else if (p.ws > 64) {
             for (int r = 0; r < nrows; r++) {
                 if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j0 + r, tid, lds);

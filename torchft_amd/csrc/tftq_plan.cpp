@@ -62,7 +62,7 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     if (vec_ok) {
         if (in_bytes <= 1024) return K_VEC8;
         if (in_bytes <= 8192) return K_VEC64;
-        if (in_bytes <= 32768) return K_VEC256;
+        return K_VEC256;  // longer than 32 KB: two passes inside the workgroup
     }
     if (s.n <= 16) return K_GEN1;
     if (s.n <= 128) return K_GEN8;
