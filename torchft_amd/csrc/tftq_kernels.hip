@@ -830,11 +830,12 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
                     w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k0 + b, ws - 1), off) + 1 + doff));
-                    w[b].w &= mask;
                 }
 #pragma unroll
-                for (int b = 0; b < 4; b++)
+                for (int b = 0; b < 4; b++) {
+                    w[b].w &= mask;
                     if (k0 + b < ws) accumulate16(acc, w[b], bcast_lane(c.r, k0 + b), bcast_lane(c.r_lo, k0 + b));
+                }
             }
             if (pass == 0) {
 #pragma unroll
@@ -1002,10 +1003,8 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
         for (int b = 0; b < PB; b++) {
             GLOBAL const u32 *pv = peer_row(p, min(lbatch * PB + b, ws - 1), off) + 1;
 #pragma unroll
-            for (int u = 0; u < UNITS; u++) {
+            for (int u = 0; u < UNITS; u++)
                 dst.w[b][u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + doff[u]));
-                dst.w[b][u].w &= padmask[u];
-            }
         }
         if (++lbatch == nb) {
             lbatch = 0;
@@ -1037,7 +1036,11 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
                 if (k < ws) {
                     const float pr = bcast_lane(cr, k), pl = bcast_lane(cl, k);
 #pragma unroll
-                    for (int u = 0; u < UNITS; u++) accumulate16(acc[u], src.w[b][u], pr, pl);
+                    for (int u = 0; u < UNITS; u++) {
+                        u32x4 w = src.w[b][u];
+                        w.w &= padmask[u];  // here, not at the load: the load must stay in flight
+                        accumulate16(acc[u], w, pr, pl);
+                    }
                 }
             }
         }
