@@ -58,6 +58,15 @@ struct InlineTable {
     Seg s[TFTQ_N_INLINE];
 };
 
+// Inline tables: XCD x works through the segments heaviest workgroups first and
+// takes a contiguous eighth of each.  Its i-th piece of work belongs to the
+// first position k with i < cum_end[x][k] and is workgroup base[x][k] + i of
+// segment seg[x][k].
+struct Dealt {
+    int32_t cum_end[8][TFTQ_N_INLINE];  // INT32_MAX past the last segment
+    struct { int32_t base, seg; } at[8][TFTQ_N_INLINE];
+};
+
 struct tftq_plan {
     int dtype;
     int esz;
@@ -68,6 +77,10 @@ struct tftq_plan {
     int64_t max_rows;
     int32_t nwg[3];
     int32_t xcd_begin[3][9];  // per stage: first workgroup of each XCD's share, balanced by bytes
+    // Plans whose segments travel in the kernel arguments deal every segment's
+    // workgroups to the 8 XCDs in equal contiguous shares instead:
+    Dealt dealt[3];
+    int32_t dealt_per_xcd[3];  // per stage: workgroups of the busiest XCD
     std::vector<Seg> segs;
     const void *device_table;  // set by the caller when nseg > TFTQ_N_INLINE
 };
@@ -81,7 +94,9 @@ struct KParams {
     int32_t nwg;
     int32_t ws;
     int32_t rank;
-    int32_t xcd_begin[9];  // workgroups [xcd_begin[x], xcd_begin[x+1]) run on XCD x
+    int32_t xcd_begin[9];  // device table: workgroups [xcd_begin[x], xcd_begin[x+1]) run on XCD x
+    int32_t per_xcd;    // workgroup ids per XCD in the grid
+    Dealt dealt;        // inline table only
     int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG general
     float div;          // reduce: 1.0 or float(ws)
     float inv_div;      // reduce: exact reciprocal when div_mode == 1

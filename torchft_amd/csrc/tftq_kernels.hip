@@ -265,32 +265,59 @@ template <> struct Elem<f16_tag> {
 // ---------------------------------------------------------------------------
 // workgroup -> (segment, first row)
 // ---------------------------------------------------------------------------
-// Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  XCD x works on
-// the contiguous range [xcd_begin[x], xcd_begin[x+1]) instead (ranges balanced by
-// bytes on the host).  The grid has 8 * (longest range) workgroups; ids past
-// the end of their range return -1.
-DEV int virtual_block(const KParams &p)
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
+// own L2.  Workgroup id b is the (b >> 3)-th piece of work of XCD b & 7.
+//
+// Inline table (at most 16 segments): XCD x takes the x-th contiguous eighth of
+// every segment's workgroups and walks the segments in p.order (heaviest
+// workgroups first).  Every XCD sees the same mix of row lengths and the last
+// workgroups to finish are light.
+// Device table: XCD x works on the contiguous range
+// [xcd_begin[x], xcd_begin[x+1]), balanced by bytes on the host.
+// Ids past the end of their XCD's work return false.
+// The kernel arguments are (KParams, InlineTable).  Indexing those by-value
+// structs with a run-time index would make the compiler copy them to private
+// memory; reading the kernel-argument segment through a constant-address-space
+// pointer keeps the accesses scalar loads.
+#define CONSTANT __attribute__((address_space(4)))
+constexpr size_t KARG_TABLE_OFF = (sizeof(KParams) + alignof(InlineTable) - 1) / alignof(InlineTable) * alignof(InlineTable);
+
+DEV const CONSTANT Seg *karg_table()
 {
-    const int x = (int)(blockIdx.x & 7);
-    const int vb = p.xcd_begin[x] + (int)(blockIdx.x >> 3);
-    return vb < p.xcd_begin[x + 1] ? vb : -1;
+    return (const CONSTANT Seg *)((const CONSTANT char *)__builtin_amdgcn_kernarg_segment_ptr() + KARG_TABLE_OFF);
 }
 
 template <bool INLINE, int STAGE>
-DEV Seg find_seg(const KParams &p, const InlineTable &inl, int vb)
+DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
 {
+    const int x = (int)(blockIdx.x & 7);
+    const int i = (int)(blockIdx.x >> 3);
     if (INLINE) {
-        int i = p.nseg - 1;
-        while (i > 0 && inl.s[i].wg_begin[STAGE] > vb) --i;
-        return inl.s[i];
+        const CONSTANT char *karg = (const CONSTANT char *)__builtin_amdgcn_kernarg_segment_ptr();
+        const CONSTANT int32_t *cum_end =
+            (const CONSTANT int32_t *)(karg + offsetof(KParams, dealt) + offsetof(Dealt, cum_end)) + x * TFTQ_N_INLINE;
+        int k = 0;
+#pragma unroll
+        for (int j = 0; j < TFTQ_N_INLINE; j++) k += i >= cum_end[j] ? 1 : 0;
+        if (k >= p.nseg) return false;
+        const CONSTANT int32_t *at =
+            (const CONSTANT int32_t *)(karg + offsetof(KParams, dealt) + offsetof(Dealt, at)) + 2 * (x * TFTQ_N_INLINE + k);
+        vb = at[0] + i;
+        const CONSTANT u32x4 *src = (const CONSTANT u32x4 *)(karg_table() + at[1]);
+        const u32x4 v[4] = {src[0], src[1], src[2], src[3]};
+        __builtin_memcpy(&s, v, sizeof(Seg));
+        return true;
     } else {
+        vb = p.xcd_begin[x] + i;
+        if (vb >= p.xcd_begin[x + 1]) return false;
         // last segment with wg_begin <= vb
         int lo = 0, hi = p.nseg - 1;
         while (lo < hi) {
             const int mid = (lo + hi + 1) >> 1;
             if (p.table[mid].wg_begin[STAGE] <= vb) lo = mid; else hi = mid - 1;
         }
-        return p.table[lo];
+        s = p.table[lo];
+        return true;
     }
 }
 
@@ -520,9 +547,9 @@ template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
-    const int vb = virtual_block(p);
-    if (vb < 0) return;
-    const Seg s = find_seg<INLINE, ST_Q>(p, inl, vb);
+    Seg s;
+    int vb;
+    if (!locate<INLINE, ST_Q>(p, inl, s, vb)) return;
     const int blk = vb - s.wg_begin[ST_Q];
     const int tid = threadIdx.x;
     switch (s.kind[ST_Q]) {
@@ -641,9 +668,9 @@ DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const InlineTable inl)
 {
-    const int vb = virtual_block(p);
-    if (vb < 0) return;
-    const Seg s = find_seg<INLINE, ST_D>(p, inl, vb);
+    Seg s;
+    int vb;
+    if (!locate<INLINE, ST_D>(p, inl, s, vb)) return;
     const int blk = vb - s.wg_begin[ST_D];
     const int tid = threadIdx.x;
     switch (s.kind[ST_D]) {
@@ -1136,9 +1163,9 @@ template <bool INLINE, bool GDIV>
 __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
-    const int vb = virtual_block(p);
-    if (vb < 0) return;
-    const Seg s = find_seg<INLINE, ST_R>(p, inl, vb);
+    Seg s;
+    int vb;
+    if (!locate<INLINE, ST_R>(p, inl, s, vb)) return;
     const int blk = vb - s.wg_begin[ST_R];
     const int tid = threadIdx.x;
     const int ndw = (s.row_bytes >> 2) - 1;
@@ -1208,6 +1235,13 @@ extern "C" int tftq_check_device(void)
 static void xcd_ranges(const tftq_plan *plan, int stage, KParams *kp)
 {
     for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = plan->xcd_begin[stage][x];
+    int longest = 0;
+    for (int x = 0; x < 8; x++) longest = std::max(longest, kp->xcd_begin[x + 1] - kp->xcd_begin[x]);
+    kp->per_xcd = longest;
+    if (plan->nseg <= TFTQ_N_INLINE) {
+        kp->dealt = plan->dealt[stage];
+        kp->per_xcd = plan->dealt_per_xcd[stage];
+    }
 }
 
 static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t packed_bytes,
@@ -1236,9 +1270,7 @@ static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t p
 
 static inline unsigned grid_of(const KParams &kp)
 {
-    int longest = 0;
-    for (int x = 0; x < 8; x++) longest = std::max(longest, kp.xcd_begin[x + 1] - kp.xcd_begin[x]);
-    return (unsigned)(8 * longest);
+    return (unsigned)(8 * kp.per_xcd);
 }
 
 template <typename T>

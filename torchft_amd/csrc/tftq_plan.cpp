@@ -149,6 +149,54 @@ static void balance_xcds(tftq_plan *p)
     }
 }
 
+// Few segments (the table travels in the kernel arguments): every XCD takes a
+// contiguous eighth of every segment, so all XCDs see the same mix of row
+// lengths, and works through the segments with the heaviest workgroups first,
+// so the last workgroups to finish are light ones.
+static void deal_to_xcds(tftq_plan *p)
+{
+    if (p->nseg > TFTQ_N_INLINE) return;
+    for (int st = 0; st < 3; st++) {
+        uint8_t ord[TFTQ_N_INLINE];
+        double w[TFTQ_N_INLINE];
+        for (int i = 0; i < p->nseg; i++) {
+            ord[i] = (uint8_t)i;
+            w[i] = wg_weight(p->segs[(size_t)i], st, p->esz, p->ws);
+        }
+        for (int i = 1; i < p->nseg; i++)  // stable insertion sort, descending weight
+            for (int j = i; j > 0 && w[ord[j]] > w[ord[j - 1]]; j--) {
+                const uint8_t t = ord[j];
+                ord[j] = ord[j - 1];
+                ord[j - 1] = t;
+            }
+        Dealt &d = p->dealt[st];
+        int64_t busiest = 0;
+        for (int x = 0; x < 8; x++) {
+            int64_t cum = 0;
+            for (int k = 0; k < TFTQ_N_INLINE; k++) {
+                if (k >= p->nseg) {
+                    d.cum_end[x][k] = INT32_MAX;
+                    d.at[x][k].base = 0;
+                    d.at[x][k].seg = 0;
+                    continue;
+                }
+                const int i = ord[k];
+                const int begin = p->segs[(size_t)i].wg_begin[st];
+                const int end = i + 1 < p->nseg ? p->segs[(size_t)i + 1].wg_begin[st] : p->nwg[st];
+                const uint64_t wgs = (uint64_t)(end - begin);
+                const int64_t lo = (int64_t)((wgs * (uint64_t)x) >> 3);
+                const int64_t hi = (int64_t)((wgs * (uint64_t)(x + 1)) >> 3);
+                d.at[x][k].base = (int32_t)(begin + lo - cum);
+                d.at[x][k].seg = i;
+                cum += hi - lo;
+                d.cum_end[x][k] = (int32_t)cum;
+            }
+            if (cum > busiest) busiest = cum;
+        }
+        p->dealt_per_xcd[st] = (int32_t)busiest;
+    }
+}
+
 extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
                                 const int64_t *shapes, const int64_t *strides, int ws,
                                 tftq_plan **out)
@@ -209,6 +257,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
     }
     for (int st = 0; st < 3; st++) p->nwg[st] = (int32_t)wg[st];
     balance_xcds(p);
+    deal_to_xcds(p);
     *out = p;
     return 0;
 }
