@@ -61,10 +61,11 @@ struct InlineTable {
 // Inline tables: XCD x works through the segments heaviest workgroups first and
 // takes a contiguous eighth of each.  Its i-th piece of work belongs to the
 // first position k with i < cum_end[x][k] and is workgroup base[x][k] + i of
-// segment seg[x][k].
+// segment seg[x][k].  Position nseg (if there is one) has seg = -1.
 struct Dealt {
-    int32_t cum_end[8][TFTQ_N_INLINE];  // INT32_MAX past the last segment
-    struct { int32_t base, seg; } at[8][TFTQ_N_INLINE];
+    int32_t cum_end[8][TFTQ_N_INLINE];  // INT32_MAX from position nseg on
+    int32_t base[8][TFTQ_N_INLINE];
+    int32_t seg[8][TFTQ_N_INLINE];
 };
 
 struct tftq_plan {

@@ -293,17 +293,27 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
     const int x = (int)(blockIdx.x & 7);
     const int i = (int)(blockIdx.x >> 3);
     if (INLINE) {
+        // One round of scalar loads fetches this XCD's three table rows; the position
+        // is then found in registers, and only the segment descriptor needs a second round.
         const CONSTANT char *karg = (const CONSTANT char *)__builtin_amdgcn_kernarg_segment_ptr();
-        const CONSTANT int32_t *cum_end =
-            (const CONSTANT int32_t *)(karg + offsetof(KParams, dealt) + offsetof(Dealt, cum_end)) + x * TFTQ_N_INLINE;
-        int k = 0;
+        const CONSTANT int32_t *d = (const CONSTANT int32_t *)(karg + offsetof(KParams, dealt)) + x * TFTQ_N_INLINE;
+        typedef int32_t Row __attribute__((ext_vector_type(TFTQ_N_INLINE)));  // one 64-byte scalar load
+        const Row cum_end = *(const CONSTANT Row *)(d + offsetof(Dealt, cum_end) / 4);
+        const Row base = *(const CONSTANT Row *)(d + offsetof(Dealt, base) / 4);
+        const Row seg = *(const CONSTANT Row *)(d + offsetof(Dealt, seg) / 4);
+        Row cum_end_ = cum_end, base_ = base, seg_ = seg;
+        // all scalar loads of this round, and the common parameters, are issued before the first wait
+        asm volatile("" : "+s"(cum_end_), "+s"(base_), "+s"(seg_) : "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
+        int b = base_[0], sg = seg_[0];
 #pragma unroll
-        for (int j = 0; j < TFTQ_N_INLINE; j++) k += i >= cum_end[j] ? 1 : 0;
-        if (k >= p.nseg) return false;
-        const CONSTANT int32_t *at =
-            (const CONSTANT int32_t *)(karg + offsetof(KParams, dealt) + offsetof(Dealt, at)) + 2 * (x * TFTQ_N_INLINE + k);
-        vb = at[0] + i;
-        const CONSTANT u32x4 *src = (const CONSTANT u32x4 *)(karg_table() + at[1]);
+        for (int j = 1; j < TFTQ_N_INLINE; j++) {
+            const bool past = i >= cum_end_[j - 1];  // cum_end is non-decreasing: the last hit wins
+            b = past ? base_[j] : b;
+            sg = past ? seg_[j] : sg;
+        }
+        if (sg < 0 || i >= cum_end_[TFTQ_N_INLINE - 1]) return false;
+        vb = b + i;
+        const CONSTANT u32x4 *src = (const CONSTANT u32x4 *)(karg_table() + sg);
         const u32x4 v[4] = {src[0], src[1], src[2], src[3]};
         __builtin_memcpy(&s, v, sizeof(Seg));
         return true;

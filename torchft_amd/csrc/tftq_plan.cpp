@@ -176,8 +176,8 @@ static void deal_to_xcds(tftq_plan *p)
             for (int k = 0; k < TFTQ_N_INLINE; k++) {
                 if (k >= p->nseg) {
                     d.cum_end[x][k] = INT32_MAX;
-                    d.at[x][k].base = 0;
-                    d.at[x][k].seg = 0;
+                    d.base[x][k] = 0;
+                    d.seg[x][k] = -1;
                     continue;
                 }
                 const int i = ord[k];
@@ -186,8 +186,8 @@ static void deal_to_xcds(tftq_plan *p)
                 const uint64_t wgs = (uint64_t)(end - begin);
                 const int64_t lo = (int64_t)((wgs * (uint64_t)x) >> 3);
                 const int64_t hi = (int64_t)((wgs * (uint64_t)(x + 1)) >> 3);
-                d.at[x][k].base = (int32_t)(begin + lo - cum);
-                d.at[x][k].seg = i;
+                d.base[x][k] = (int32_t)(begin + lo - cum);
+                d.seg[x][k] = i;
                 cum += hi - lo;
                 d.cum_end[x][k] = (int32_t)cum;
             }
