@@ -254,7 +254,7 @@ def main() -> int:
     # The roofline entry is for the kernel that takes the largest share of the step.
     # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE (x2.000,
     # calibrated on a 256 MiB copy) + WRITE_SIZE (x1.000); profiles/cfg3_bf16_ws8_hbm_traffic.md
-    measured_traffic = {"quantize": 654869000, "reduce": 248633000, "dequantize": 661127000}
+    measured_traffic = {"quantize": 654942000, "reduce": 247438000, "dequantize": 660774000}
     dominant = max(stages, key=lambda k: stages[k]["us"])
     roofline = {"bound": "hbm", "kernel": "k_" + dominant, "achieved": stages[dominant]["GBs"],
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": stages[dominant]["frac"],
