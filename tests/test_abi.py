@@ -78,7 +78,8 @@ def test_plan_sizes_and_table():
     shapes = [(3, 5)] * 40
     rc, h = _plan(0, shapes, [(5, 1)] * 40, 4)
     assert rc == 0
-    assert L.tftq_plan_table_bytes(h) == 40 * 64
+    # 40 descriptors of 64 bytes, then the per-stage lookup tables
+    assert L.tftq_plan_table_bytes(h) > 40 * 64 and L.tftq_plan_table_bytes(h) % 8 == 0
     assert L.tftq_plan_table_host(h)
     assert L.tftq_plan_max_rows(h) == 4
     # no device table bound yet: compute entry points refuse instead of launching

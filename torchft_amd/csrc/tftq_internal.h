@@ -58,14 +58,36 @@ struct InlineTable {
     Seg s[TFTQ_N_INLINE];
 };
 
-// Inline tables: XCD x works through the segments heaviest workgroups first and
-// takes a contiguous eighth of each.  Its i-th piece of work belongs to the
-// first position k with i < cum_end[x][k] and is workgroup base[x][k] + i of
-// segment seg[x][k].  Position nseg (if there is one) has seg = -1.
+// Inline tables (at most TFTQ_N_INLINE segments): XCD x works through the
+// segments in the stage's work order (reduce: heaviest workgroups first;
+// quantize and dequantize: list order) and takes a contiguous eighth of each.
+// Its i-th piece of work belongs to the first position k with
+// i < cum_end[x][k] and is workgroup base[x][k] + i of segment seg[x][k].
+// Position nseg (if there is one) has seg = -1.
 struct Dealt {
     int32_t cum_end[8][TFTQ_N_INLINE];  // INT32_MAX from position nseg on
     int32_t base[8][TFTQ_N_INLINE];
     int32_t seg[8][TFTQ_N_INLINE];
+};
+
+// Device tables (longer lists).  Per stage, workgroup numbers are handed out to
+// the segments in the stage's work order; chunks of 2^chunk_shift consecutive
+// workgroups go to the XCDs in turn, so all XCDs work down the same list.  A chunk is about 1/64 of an XCD's work and at
+// least 16 workgroups: large enough that an XCD touches only its own pages of a
+// big tensor, small enough that the XCDs finish together.  The device table holds
+//   Seg      segs[nseg]                    in list order
+//   SortEnt  sorted[3][nseg]               per stage, in workgroup order
+//   MapEnt   map[3][...]                   per stage: bucket of 2^shift workgroups -> position
+// and a workgroup finds its segment with one load of map[b], map[b+1] and, only
+// if those differ, a binary search of sorted[] between the two positions.
+struct SortEnt { int32_t begin, seg; };  // first workgroup of the segment, index into segs[]
+struct MapEnt { int32_t pos, seg; };     // position in sorted[] that holds workgroup b << shift
+struct TableIndex {
+    int64_t sorted_off;  // bytes from the start of the device table
+    int64_t map_off;
+    int32_t shift;
+    int32_t chunk_shift;
+    int32_t per_xcd;     // workgroup ids per XCD in the grid
 };
 
 struct tftq_plan {
@@ -77,13 +99,12 @@ struct tftq_plan {
     int64_t output_size;
     int64_t max_rows;
     int32_t nwg[3];
-    int32_t xcd_begin[3][9];  // per stage: first workgroup of each XCD's share, balanced by bytes
-    // Plans whose segments travel in the kernel arguments deal every segment's
-    // workgroups to the 8 XCDs in equal contiguous shares instead:
-    Dealt dealt[3];
-    int32_t dealt_per_xcd[3];  // per stage: workgroups of the busiest XCD
+    Dealt dealt[3];            // inline table only
+    int32_t dealt_per_xcd[3];  // inline table only: workgroups of the busiest XCD
+    TableIndex index[3];       // device table only
     std::vector<Seg> segs;
-    const void *device_table;  // set by the caller when nseg > TFTQ_N_INLINE
+    std::vector<uint8_t> blob;  // host image of the device table (nseg > TFTQ_N_INLINE)
+    const void *device_table;   // set by the caller when nseg > TFTQ_N_INLINE
 };
 
 // Kernel parameters common to the three stages.
@@ -95,8 +116,11 @@ struct KParams {
     int32_t nwg;
     int32_t ws;
     int32_t rank;
-    int32_t xcd_begin[9];  // device table: workgroups [xcd_begin[x], xcd_begin[x+1]) run on XCD x
     int32_t per_xcd;    // workgroup ids per XCD in the grid
+    int32_t map_shift;  // device table only, as are the next three
+    int32_t chunk_shift;
+    int64_t sorted_off;
+    int64_t map_off;
     Dealt dealt;        // inline table only
     int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG general
     float div;          // reduce: 1.0 or float(ws)

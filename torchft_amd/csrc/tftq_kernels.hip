@@ -269,12 +269,14 @@ template <> struct Elem<f16_tag> {
 // own L2.  Workgroup id b is the (b >> 3)-th piece of work of XCD b & 7.
 //
 // Inline table (at most 16 segments): XCD x takes the x-th contiguous eighth of
-// every segment's workgroups and walks the segments in p.order (heaviest
-// workgroups first).  Every XCD sees the same mix of row lengths and the last
-// workgroups to finish are light.
-// Device table: XCD x works on the contiguous range
-// [xcd_begin[x], xcd_begin[x+1]), balanced by bytes on the host.
+// every segment's workgroups and walks the segments in the stage's work order
+// (reduce: heaviest workgroups first, so that every XCD sees the same mix of
+// row lengths and the last workgroups to finish are light).
+// Device table (longer lists): workgroup numbers follow the segments in the
+// stage's work order, chunks of consecutive numbers go to the XCDs in turn, and
+// a bucket map plus a short binary search lead from the number to the segment.
 // Ids past the end of their XCD's work return false.
+//
 // The kernel arguments are (KParams, InlineTable).  Indexing those by-value
 // structs with a run-time index would make the compiler copy them to private
 // memory; reading the kernel-argument segment through a constant-address-space
@@ -318,15 +320,29 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
         __builtin_memcpy(&s, v, sizeof(Seg));
         return true;
     } else {
-        vb = p.xcd_begin[x] + i;
-        if (vb >= p.xcd_begin[x + 1]) return false;
-        // last segment with wg_begin <= vb
-        int lo = 0, hi = p.nseg - 1;
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (p.table[mid].wg_begin[STAGE] <= vb) lo = mid; else hi = mid - 1;
+        // everything the first steps need from the kernel arguments in one round of scalar loads
+        asm volatile("" ::"s"(p.table), "s"(p.map_off), "s"(p.sorted_off), "s"(p.map_shift), "s"(p.chunk_shift), "s"(p.nwg),
+                     "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
+        // chunks of 2^chunk_shift consecutive workgroups go to the XCDs in turn
+        const int cs = p.chunk_shift;
+        vb = ((((i >> cs) << 3) + x) << cs) + (i & ((1 << cs) - 1));
+        if (vb >= p.nwg) return false;
+        const uint64_t tab = (uint64_t)p.table;
+        typedef int32_t MapPair __attribute__((ext_vector_type(4), aligned(8)));
+        const MapPair m = *(const CONSTANT MapPair *)(tab + (uint64_t)p.map_off +
+                                                      (uint64_t)(vb >> p.map_shift) * sizeof(MapEnt));
+        int lo = m.x, sg = m.y, hi = m.z;
+        if (lo != hi) {  // last position whose first workgroup is <= vb
+            const CONSTANT SortEnt *sorted = (const CONSTANT SortEnt *)(tab + (uint64_t)p.sorted_off);
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (sorted[mid].begin <= vb) lo = mid; else hi = mid - 1;
+            }
+            sg = sorted[lo].seg;
         }
-        s = p.table[lo];
+        const CONSTANT u32x4 *src = (const CONSTANT u32x4 *)(tab + (uint64_t)sg * sizeof(Seg));
+        const u32x4 v[4] = {src[0], src[1], src[2], src[3]};
+        __builtin_memcpy(&s, v, sizeof(Seg));
         return true;
     }
 }
@@ -1242,15 +1258,19 @@ extern "C" int tftq_check_device(void)
                : TFTQ_E_ARCH;
 }
 
-static void xcd_ranges(const tftq_plan *plan, int stage, KParams *kp)
+static void work_mapping(const tftq_plan *plan, int stage, KParams *kp)
 {
-    for (int x = 0; x <= 8; x++) kp->xcd_begin[x] = plan->xcd_begin[stage][x];
-    int longest = 0;
-    for (int x = 0; x < 8; x++) longest = std::max(longest, kp->xcd_begin[x + 1] - kp->xcd_begin[x]);
-    kp->per_xcd = longest;
     if (plan->nseg <= TFTQ_N_INLINE) {
         kp->dealt = plan->dealt[stage];
         kp->per_xcd = plan->dealt_per_xcd[stage];
+        kp->map_shift = kp->chunk_shift = 0;
+        kp->sorted_off = kp->map_off = 0;
+    } else {
+        kp->per_xcd = plan->index[stage].per_xcd;
+        kp->map_shift = plan->index[stage].shift;
+        kp->chunk_shift = plan->index[stage].chunk_shift;
+        kp->sorted_off = plan->index[stage].sorted_off;
+        kp->map_off = plan->index[stage].map_off;
     }
 }
 
@@ -1268,7 +1288,7 @@ static int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t p
     kp->nseg = plan->nseg;
     kp->nwg = plan->nwg[stage];
     kp->ws = plan->ws;
-    xcd_ranges(plan, stage, kp);
+    work_mapping(plan, stage, kp);
     kp->rank = 0;
     kp->div_mode = 0;
     kp->div = 1.0f;

@@ -9,7 +9,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <new>
+#include <vector>
 
 #include "../../include/tftq.h"
 #include "tftq_internal.h"
@@ -110,65 +112,37 @@ static double wg_weight(const Seg &s, int st, int esz, int ws)
     return rows * ((double)s.n * esz + (double)s.row_bytes);
 }
 
-// Workgroup ids are dealt round-robin to the 8 XCDs by the hardware; the
-// kernels turn that into one contiguous range of workgroups per XCD.  Choose
-// the ranges so that every XCD moves about the same number of bytes (rows of
-// different tensors differ in length by up to 3.5x in one call).
-static void balance_xcds(tftq_plan *p)
+// The order in which a stage works through the segments.  Reduce: by workgroup
+// weight, heaviest first (equal weights keep the list order), so that the last
+// workgroups to finish are light; its weights differ by orders of magnitude
+// within one list.  Quantize and dequantize keep the list order: their
+// workgroups are all of similar weight, and sorting them measured slower.
+static void work_order(const tftq_plan *p, int st, std::vector<int32_t> &ord)
 {
-    for (int st = 0; st < 3; st++) {
-        int32_t *xb = p->xcd_begin[st];
-        const int nwg = p->nwg[st];
-        double total = 0;
-        for (int i = 0; i < p->nseg; i++) {
-            const Seg &s = p->segs[(size_t)i];
-            const int end = i + 1 < p->nseg ? p->segs[(size_t)i + 1].wg_begin[st] : nwg;
-            total += (double)(end - s.wg_begin[st]) * wg_weight(s, st, p->esz, p->ws);
-        }
-        xb[0] = 0;
-        int x = 1;
-        double cum = 0;
-        for (int i = 0; i < p->nseg && x < 8; i++) {
-            const Seg &s = p->segs[(size_t)i];
-            const int begin = s.wg_begin[st];
-            const int end = i + 1 < p->nseg ? p->segs[(size_t)i + 1].wg_begin[st] : nwg;
-            const double w = wg_weight(s, st, p->esz, p->ws);
-            if (end == begin || w <= 0) continue;
-            const double seg_total = (double)(end - begin) * w;
-            while (x < 8 && cum + seg_total >= total * x / 8.0) {
-                double k = (total * x / 8.0 - cum) / w;  // workgroups of this segment before the cut
-                int cut = begin + (int)(k + 0.5);
-                if (cut < xb[x - 1]) cut = xb[x - 1];
-                if (cut > end) cut = end;
-                xb[x++] = cut;
-            }
-            cum += seg_total;
-        }
-        while (x <= 8) xb[x++] = nwg;
-        xb[8] = nwg;
+    std::vector<double> w((size_t)p->nseg);
+    ord.resize((size_t)p->nseg);
+    for (int i = 0; i < p->nseg; i++) {
+        ord[(size_t)i] = i;
+        w[(size_t)i] = wg_weight(p->segs[(size_t)i], st, p->esz, p->ws);
     }
+    if (st != ST_R) return;
+    std::stable_sort(ord.begin(), ord.end(), [&](int32_t a, int32_t b) { return w[(size_t)a] > w[(size_t)b]; });
 }
 
-// Few segments (the table travels in the kernel arguments): every XCD takes a
+// Few segments (the table travels in the kernel arguments).  Workgroup ids are
+// dealt round-robin to the 8 XCDs by the hardware; here every XCD takes a
 // contiguous eighth of every segment, so all XCDs see the same mix of row
-// lengths, and works through the segments with the heaviest workgroups first,
-// so the last workgroups to finish are light ones.
-static void deal_to_xcds(tftq_plan *p)
+// lengths, and works through the segments in work_order().
+static void deal_to_xcds(tftq_plan *p, const int32_t (*wgs)[3])
 {
-    if (p->nseg > TFTQ_N_INLINE) return;
     for (int st = 0; st < 3; st++) {
-        uint8_t ord[TFTQ_N_INLINE];
-        double w[TFTQ_N_INLINE];
-        for (int i = 0; i < p->nseg; i++) {
-            ord[i] = (uint8_t)i;
-            w[i] = wg_weight(p->segs[(size_t)i], st, p->esz, p->ws);
+        int32_t begin = 0;
+        for (int i = 0; i < p->nseg; i++) {  // workgroup numbers in list order
+            p->segs[(size_t)i].wg_begin[st] = begin;
+            begin += wgs[i][st];
         }
-        for (int i = 1; i < p->nseg; i++)  // stable insertion sort, descending weight
-            for (int j = i; j > 0 && w[ord[j]] > w[ord[j - 1]]; j--) {
-                const uint8_t t = ord[j];
-                ord[j] = ord[j - 1];
-                ord[j - 1] = t;
-            }
+        std::vector<int32_t> ord;
+        work_order(p, st, ord);
         Dealt &d = p->dealt[st];
         int64_t busiest = 0;
         for (int x = 0; x < 8; x++) {
@@ -180,13 +154,11 @@ static void deal_to_xcds(tftq_plan *p)
                     d.seg[x][k] = -1;
                     continue;
                 }
-                const int i = ord[k];
-                const int begin = p->segs[(size_t)i].wg_begin[st];
-                const int end = i + 1 < p->nseg ? p->segs[(size_t)i + 1].wg_begin[st] : p->nwg[st];
-                const uint64_t wgs = (uint64_t)(end - begin);
-                const int64_t lo = (int64_t)((wgs * (uint64_t)x) >> 3);
-                const int64_t hi = (int64_t)((wgs * (uint64_t)(x + 1)) >> 3);
-                d.base[x][k] = (int32_t)(begin + lo - cum);
+                const int i = ord[(size_t)k];
+                const uint64_t n = (uint64_t)wgs[i][st];
+                const int64_t lo = (int64_t)((n * (uint64_t)x) >> 3);
+                const int64_t hi = (int64_t)((n * (uint64_t)(x + 1)) >> 3);
+                d.base[x][k] = (int32_t)(p->segs[(size_t)i].wg_begin[st] + lo - cum);
                 d.seg[x][k] = i;
                 cum += hi - lo;
                 d.cum_end[x][k] = (int32_t)cum;
@@ -195,6 +167,63 @@ static void deal_to_xcds(tftq_plan *p)
         }
         p->dealt_per_xcd[st] = (int32_t)busiest;
     }
+}
+
+// Many segments: the image of the device table (layout in tftq_internal.h).
+static int build_table(tftq_plan *p, const int32_t (*wgs)[3])
+{
+    const size_t nseg = (size_t)p->nseg;
+    std::vector<SortEnt> sorted[3];
+    std::vector<MapEnt> map[3];
+    for (int st = 0; st < 3; st++) {
+        std::vector<int32_t> ord;
+        work_order(p, st, ord);
+        sorted[st].resize(nseg);
+        int32_t begin = 0;
+        for (size_t k = 0; k < nseg; k++) {  // workgroup numbers in sorted order
+            const int32_t i = ord[k];
+            p->segs[(size_t)i].wg_begin[st] = begin;
+            sorted[st][k] = SortEnt{begin, i};
+            begin += wgs[i][st];
+        }
+        const int64_t nwg = p->nwg[st];
+        int shift = 0;
+        while ((nwg >> shift) > 4 * (int64_t)nseg) shift++;
+        const int64_t nb = (nwg >> shift) + 1;  // buckets; map[] has one more entry
+        map[st].resize((size_t)nb + 1);
+        size_t k = 0;
+        for (int64_t b = 0; b <= nb; b++) {
+            const int64_t w = b << shift;
+            if (w >= nwg) {
+                k = nseg - 1;
+            } else {
+                while (k + 1 < nseg && sorted[st][k + 1].begin <= w) k++;
+            }
+            map[st][(size_t)b] = MapEnt{(int32_t)k, sorted[st][k].seg};
+        }
+        p->index[st].shift = shift;
+        int cs = 4;
+        while (cs < 20 && (nwg >> (cs + 1)) >= 8 * 64) cs++;
+        p->index[st].chunk_shift = cs;
+        const int64_t turns = (nwg + ((int64_t)8 << cs) - 1) / ((int64_t)8 << cs);
+        p->index[st].per_xcd = (int32_t)(turns << cs);
+    }
+    size_t bytes = nseg * sizeof(Seg);
+    for (int st = 0; st < 3; st++) {
+        p->index[st].sorted_off = (int64_t)bytes;
+        bytes += nseg * sizeof(SortEnt);
+    }
+    for (int st = 0; st < 3; st++) {
+        p->index[st].map_off = (int64_t)bytes;
+        bytes += map[st].size() * sizeof(MapEnt);
+    }
+    p->blob.resize(bytes);
+    memcpy(p->blob.data(), p->segs.data(), nseg * sizeof(Seg));
+    for (int st = 0; st < 3; st++) {
+        memcpy(p->blob.data() + p->index[st].sorted_off, sorted[st].data(), nseg * sizeof(SortEnt));
+        memcpy(p->blob.data() + p->index[st].map_off, map[st].data(), map[st].size() * sizeof(MapEnt));
+    }
+    return 0;
 }
 
 extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
@@ -227,6 +256,14 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         return rc;
     }
     int64_t wg[3] = {0, 0, 0};
+    std::vector<int32_t> wgs_flat;
+    try {
+        wgs_flat.resize((size_t)n_tensors * 3);
+    } catch (...) {
+        delete p;
+        return TFTQ_E_NOMEM;
+    }
+    int32_t (*wgs)[3] = (int32_t (*)[3])wgs_flat.data();  // workgroups per segment and stage
     for (int i = 0; i < n_tensors; i++) {
         Seg &s = p->segs[(size_t)i];
         memset(&s, 0, sizeof(s));
@@ -246,18 +283,23 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         s.reduce_rows_per_team = (uint8_t)pick_reduce_rows(s, ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
-            s.wg_begin[st] = (int32_t)wg[st];
-            const int rows_per_wg = rows_per_wg_of(s, st);
-            wg[st] += cdiv64(rows[st], rows_per_wg);
-            if (wg[st] > INT32_MAX - 16) {
+            const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st));
+            wgs[i][st] = (int32_t)n;
+            wg[st] += n;
+            if (wg[st] > INT32_MAX - 4096) {
                 delete p;
                 return TFTQ_E_SHAPE;
             }
         }
     }
     for (int st = 0; st < 3; st++) p->nwg[st] = (int32_t)wg[st];
-    balance_xcds(p);
-    deal_to_xcds(p);
+    try {
+        if (p->nseg <= TFTQ_N_INLINE) deal_to_xcds(p, wgs);
+        else build_table(p, wgs);
+    } catch (...) {
+        delete p;
+        return TFTQ_E_NOMEM;
+    }
     *out = p;
     return 0;
 }
@@ -271,12 +313,13 @@ extern "C" int64_t tftq_plan_max_rows(const tftq_plan *plan) { return plan ? pla
 extern "C" int64_t tftq_plan_table_bytes(const tftq_plan *plan)
 {
     if (!plan) return -1;
-    return plan->nseg > TFTQ_N_INLINE ? (int64_t)plan->nseg * (int64_t)sizeof(Seg) : 0;
+    return plan->nseg > TFTQ_N_INLINE ? (int64_t)plan->blob.size() : 0;
 }
 
 extern "C" const void *tftq_plan_table_host(const tftq_plan *plan)
 {
-    return plan ? (const void *)plan->segs.data() : nullptr;
+    if (!plan) return nullptr;
+    return plan->nseg > TFTQ_N_INLINE ? (const void *)plan->blob.data() : (const void *)plan->segs.data();
 }
 
 extern "C" int tftq_plan_set_device_table(tftq_plan *plan, const void *device_table)
