@@ -4,10 +4,12 @@ orchestration of the quantized collectives on a single GPU.
 Every rank is a thread (as in the reference's own collective tests,
 torchft/process_group_test.py:863-898) and all ranks share the one device.  Only
 the two collectives the quantized path needs are provided, with the semantics
-pinned by process_group_test.py:175-215 (all-gather) and :255-296 (all-to-all):
+pinned by process_group_test.py:175-215 (all-gather) and :255-296 (all-to-all),
+plus a SUM all-reduce for the unquantized branch of the managed all-reduce:
 
     alltoall_base(out, inp):                      out[p] on rank r  =  inp[r] of rank p
     allgather_into_tensor_coalesced([out], [inp]): out[p] on rank r =  inp of rank p
+    allreduce([t]):                               t on every rank  =  sum_p t of rank p, p ascending
 
 The copies are queued on each rank's current stream behind events of the
 producers, so nothing blocks the host except the thread barrier that publishes
@@ -86,3 +88,15 @@ class SimProcessGroup:
         out = output_tensors[0]
         return self._exchange(
             input_tensors[0], lambda p, src: out[p].copy_(src.reshape(out[p].shape), non_blocking=True))
+
+    def allreduce(self, tensors, opts=None):
+        assert len(tensors) == 1
+        t = tensors[0]
+        acc = torch.zeros_like(t)
+
+        def pull(p, src):
+            acc.add_(src)
+
+        work = self._exchange(t.clone(), pull)
+        t.copy_(acc)
+        return work

@@ -1,0 +1,210 @@
+"""The callers of the quantized all-reduce: one managed all-reduce of a tensor and
+DiLoCo's bucketised averaging of pseudo-gradients.
+
+Data path of ``Manager.allreduce`` (torchft/manager.py:386-467) and of
+``_StreamingDiLoCoFragment._bucketize_and_allreduce`` /
+``_allreduce_per_param`` (torchft/local_sgd.py:489-567), without the manager's
+quorum, error tracking and healing: what is left is which tensors go through
+:func:`torchft_amd.collectives.allreduce_quantized`, with which reduce op, on
+which stream, and what is done to the result.
+
+* ``allreduce`` zeroes the tensor of a replica that is not participating, turns
+  AVG into SUM for the collective and divides by the number of participants in
+  a continuation of the collective's future (manager.py:419-456).  With
+  ``should_quantize`` the list ``[tensor]`` goes to ``allreduce_quantized`` on
+  the current stream (manager.py:432-439); a 1-D tensor is quantized as rows of
+  one column (quantization.py:487-488), 8 packed bytes per element.
+* ``bucketize_and_allreduce`` packs the tensors into flat zero-initialised
+  buffers of at most ``bucket_size_bytes``, reduces each buffer and copies the
+  result back in the continuation (local_sgd.py:499-556).
+
+``row_width`` is an addition with no counterpart in the reference: the flat
+bucket is handed to the all-reduce as a 2-D view ``[rows, row_width]``, so that
+quantization keeps one scale per ``row_width`` elements (``row_width + 4`` packed
+bytes per row) instead of one per element.  It changes the quantization
+granularity, hence the values, and is off by default.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Callable
+
+import torch
+from torch.distributed import ReduceOp
+from torch.distributed.distributed_c10d import AllreduceOptions
+
+from .collectives import allreduce_quantized
+
+
+class _Completed:
+    """What a continuation is called with: the value the chain has reached."""
+
+    def __init__(self, value: Any) -> None:
+        self._value = value
+
+    def wait(self) -> Any:
+        return self._value
+
+    def value(self) -> Any:
+        return self._value
+
+
+class _ChainFuture:
+    """The future of a :class:`_ChainedWork`: ``then`` appends to the work's chain,
+    so that the continuation runs on the work's stream like the ones before it."""
+
+    def __init__(self, work: "_ChainedWork") -> None:
+        self._work = work
+
+    def then(self, callback: Callable[[Any], Any]) -> "_ChainFuture":
+        self._work._then(lambda value: callback(_Completed(value)))
+        return self
+
+    def wait(self) -> Any:
+        return self._work._tail.wait()
+
+    def value(self) -> Any:
+        return self._work._tail.value()
+
+
+class _ChainedWork:
+    """The collective's work plus the continuations that finish the tensor.
+
+    Every continuation runs with the stream that was current when the work was
+    created, after a dependency on the collective (manager.py:1214-1227), in
+    the order in which it was added."""
+
+    def __init__(self, work: Any, value: Any) -> None:
+        self._work = work
+        self._stream = torch.cuda.current_stream() if torch.cuda.is_available() else None
+        self._tail: torch.futures.Future = work.get_future().then(lambda fut: value)
+
+    def _then(self, callback: Callable[[Any], Any]) -> None:
+        stream = self._stream
+
+        def run(fut: torch.futures.Future) -> Any:
+            if stream is None:
+                return callback(fut.wait())
+            with torch.cuda.stream(stream):
+                return callback(fut.wait())
+
+        self._tail = self._tail.then(run)
+
+    def wait(self, timeout=None) -> bool:
+        self._work.wait()
+        self._tail.wait()
+        return True
+
+    def get_future(self) -> _ChainFuture:
+        return _ChainFuture(self)
+
+
+def allreduce(
+    tensor: torch.Tensor,
+    process_group: Any,
+    num_participants: int,
+    is_participating: bool = True,
+    should_quantize: bool = False,
+    reduce_op: ReduceOp = ReduceOp.AVG,
+):
+    """
+    All-reduce ``tensor`` in place over ``process_group`` and scale it by
+    ``1 / num_participants`` when ``reduce_op`` is AVG (manager.py:386-456).
+
+    Returns a work whose future completes with the tensor.  The result is in
+    ``tensor`` once the work has been waited on, in stream order of the stream
+    that was current at the call.
+    """
+    if not is_participating:
+        tensor.zero_()  # manager.py:419-420
+
+    pg_reduce_op = reduce_op
+    if reduce_op == ReduceOp.AVG:
+        if not torch.is_floating_point(tensor):
+            raise ValueError("average reduce op is only supported for floating point tensors")
+        pg_reduce_op = ReduceOp.SUM  # manager.py:422-429
+
+    if should_quantize:
+        work = allreduce_quantized([tensor], pg_reduce_op, process_group, torch.cuda.current_stream())
+    else:
+        opts = AllreduceOptions()
+        opts.reduceOp = pg_reduce_op
+        work = process_group.allreduce([tensor], opts)
+
+    chained = _ChainedWork(work, tensor)
+
+    def normalize(value: torch.Tensor) -> torch.Tensor:
+        if reduce_op == ReduceOp.AVG:
+            value /= num_participants  # manager.py:450-452
+        return value
+
+    chained._then(normalize)
+    return chained
+
+
+def allreduce_per_param(grads: dict, allreduce_fn: Callable[[torch.Tensor], Any]) -> list:
+    """One all-reduce per pseudo-gradient (local_sgd.py:489-497)."""
+    return [allreduce_fn(g) for g in grads.values()]
+
+
+def bucketize_and_allreduce(
+    tensors: list,
+    bucket_size_bytes: int,
+    allreduce_fn: Callable[[torch.Tensor], Any],
+    row_width: int | None = None,
+) -> list:
+    """
+    All-reduce ``tensors`` through flat buffers of at most ``bucket_size_bytes``
+    (local_sgd.py:499-556) and return the works; each tensor holds its reduced
+    values once its bucket's work has been waited on.
+
+    The packing is the reference's, including its corner: the running offset
+    advances by the bucket capacity, not by what was packed (:553), so when a
+    tensor does not fit into the space left in a bucket the loop can end before
+    the last tensors have been packed; those keep their local values.  A
+    bucket capacity that is a multiple of every tensor's size, or larger than
+    the whole list, avoids it.
+
+    ``allreduce_fn(flat)`` is, for example,
+    ``lambda t: allreduce(t, pg, n, should_quantize=True)``.
+    """
+    works: list = []
+    if not tensors:
+        return works
+
+    total_size = sum(t.numel() for t in tensors)
+    dtype, device = tensors[0].dtype, tensors[0].device
+    per_bucket = bucket_size_bytes // tensors[0].element_size()
+    assert per_bucket > 0, "bucket_size_bytes is smaller than one element"
+
+    offset = 0
+    flat_index = 0
+    while offset < total_size:
+        chunk_size = min(per_bucket, total_size - offset)
+        alloc = chunk_size
+        if row_width:
+            alloc = -(-chunk_size // row_width) * row_width  # whole rows; the tail stays zero
+        flat_buffer = torch.zeros(alloc, dtype=dtype, device=device)
+
+        pack_offset = 0
+        bucket_tensors: list = []
+        for t in tensors[flat_index:]:
+            numel = t.numel()
+            if pack_offset + numel > chunk_size:
+                break
+            flat_buffer[pack_offset:pack_offset + numel].copy_(t.view(-1))
+            bucket_tensors.append((t, pack_offset, numel))
+            pack_offset += numel
+            flat_index += 1
+
+        work = allreduce_fn(flat_buffer.view(-1, row_width) if row_width else flat_buffer)
+
+        def unpack(fut, bucket_tensors=bucket_tensors, flat_buffer=flat_buffer):
+            for t, pack_offset, numel in bucket_tensors:
+                t.copy_(flat_buffer[pack_offset:pack_offset + numel].view_as(t))
+            return []
+
+        work.get_future().then(unpack)
+        works.append(work)
+        offset += chunk_size
+    return works
