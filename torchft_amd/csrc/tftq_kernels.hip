@@ -635,7 +635,7 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
         return;
     }
     constexpr int EPV = Elem<T>::EPV;
-    constexpr int DV = 4;
+    constexpr int DV = 8;  // loads in flight per lane (4: 1.3 % slower on 4096-column bf16 rows)
     const int nvec = s.n / EPV;
     GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
     // the few columns after the last whole vector, one element per lane

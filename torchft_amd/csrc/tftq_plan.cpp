@@ -82,20 +82,12 @@ static uint8_t pick_reduce_kind(const Seg &s)
     return K_GEN256;
 }
 
-// Reduce: a wide team works through several consecutive short rows, prefetching
-// the next one; about 32 KB of peer rows per team (measured best on MI355X:
-// more rows per team leave too few workgroups to balance the CUs).
-static int reduce_team_bytes() { return 32 * 1024; }
-
-static int pick_reduce_rows(const Seg &s, int ws)
-{
-    if (s.kind[ST_R] != K_GEN256 && s.kind[ST_R] != K_GEN64) return 1;
-    const int64_t per_row = (int64_t)s.row_bytes * ws;
-    int64_t r = (reduce_team_bytes() + per_row / 2) / per_row;
-    if (r < 1) r = 1;
-    if (r > 16) r = 16;
-    return (int)r;
-}
+// Reduce: rows one team works through, prefetching the next row while it
+// finishes the current one.  The kernels support it; one row per team measured
+// fastest on MI355X for every row length (1024-column rows, ws 8: 44 us with
+// one row, 49 / 53 / 67 us with 2 / 4 / 8), because independent workgroups keep
+// more loads in flight than one team's pipeline does.
+static int pick_reduce_rows(const Seg &, int) { return 1; }
 
 static int rows_per_wg_of(const Seg &s, int st)
 {
