@@ -260,6 +260,31 @@ def test_group_sizes(q, oracle, ws, op):
     full_check(q, oracle, peers, ws, op, ranks)
 
 
+@pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (16, ReduceOp.AVG), (24, ReduceOp.SUM),
+                                   (40, ReduceOp.AVG)])
+def test_short_rows_all_team_sizes(q, oracle, ws, op):
+    """Rows of 17 ... 600 columns: teams of 8, 16 and 32 lanes in reduce, several rows per
+    wavefront, row counts that leave the last workgroup partly empty, group sizes below and
+    above the team size, and some rows whose scale needs the plain divide."""
+    g = torch.Generator().manual_seed(100 + ws)
+    cols = [17, 20, 36, 64, 100, 128, 131, 200, 256, 257, 300, 500, 512, 513, 600]
+    rows = [ws * 3 + 5, 45, ws + 1]
+    shapes = [(rows[i % 3], c) for i, c in enumerate(cols)]
+    peers = []
+    for p in range(ws):
+        ts = []
+        for r, c in shapes:
+            x = torch.randn(r, c, generator=g) * (1 + p % 3)
+            x[1] *= 1e-30  # row scale beyond 2^64: the exact fallback inside a shared wavefront
+            x[min(3, r - 1)] = 0.0
+            ts.append(x)
+        peers.append(ts)
+    ranks = None if ws <= 8 else [0, ws - 1]
+    full_check(q, oracle, peers, ws, op, ranks)
+    half = [[t.to(torch.bfloat16) for t in ts] for ts in peers]
+    full_check(q, oracle, half, ws, op, [ws // 2])
+
+
 def test_long_rows(q, oracle):
     """Rows longer than the register-resident paths hold: 20000 and 70000 columns."""
     g = torch.Generator().manual_seed(21)

@@ -22,12 +22,18 @@ enum : uint8_t {
     K_GEN64 = 6,   // one wavefront per row
     K_GEN256 = 7,  // one workgroup per row (reduce only)
     K_COL1 = 8,    // rows of a single column (1-D tensors): 4 rows per lane, 1024 per workgroup
+    K_GEN16 = 9,   // 16 lanes per row (reduce only)
+    K_GEN32 = 10,  // 32 lanes per row (reduce only)
+    K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
+    K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
 };
 
 static inline int tftq_team_of(uint8_t kind)
 {
     switch (kind) {
     case K_VEC8: case K_GEN8: return 8;
+    case K_GEN16: case K_VEC16: return 16;
+    case K_GEN32: case K_VEC32: return 32;
     case K_VEC64: case K_GEN64: return 64;
     case K_VEC256: case K_GEN256: return 256;
     case K_GEN1: return 1;

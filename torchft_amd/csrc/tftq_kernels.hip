@@ -30,6 +30,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "../../include/tftq.h"
 #include "tftq_internal.h"
@@ -85,6 +86,20 @@ DEV float bcast_lane(float v, int lane)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
+// v of lane k of the caller's team (k uniform).  Teams of whole wavefronts hold
+// the same values in every wavefront and read lane k; smaller teams go through
+// the LDS crossbar.
+template <int TEAM>
+DEV float team_bcast(float v, int k)
+{
+    if constexpr (TEAM >= 64) {
+        return bcast_lane(v, k);
+    } else {
+        const int base = (int)(threadIdx.x & 63u) & ~(TEAM - 1);
+        return __int_as_float(__builtin_amdgcn_ds_bpermute((base + k) << 2, __float_as_int(v)));
+    }
+}
+
 // max over the TEAM lanes that share a row; every lane of the team gets it.
 // lds: 4 floats per workgroup, used by 256-lane teams only.
 template <int TEAM>
@@ -95,11 +110,12 @@ DEV float team_max(float v, float *lds)
         v = fmaxf(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
         v = fmaxf(v, dpp_mov<0x141>(v));  // row_half_mirror
     }
-    if (TEAM >= 64) {
-        v = fmaxf(v, dpp_mov<0x140>(v));  // row_mirror: all 16 lanes of a row agree
+    if (TEAM >= 16) v = fmaxf(v, dpp_mov<0x140>(v));  // row_mirror: all 16 lanes of a row agree
+    if (TEAM >= 32) {
         const float a = bcast_lane(v, 0), b = bcast_lane(v, 16);
         const float c = bcast_lane(v, 32), d = bcast_lane(v, 48);
-        v = fmaxf(fmaxf(a, b), fmaxf(c, d));
+        if (TEAM == 32) v = (threadIdx.x & 32) ? fmaxf(c, d) : fmaxf(a, b);
+        else v = fmaxf(fmaxf(a, b), fmaxf(c, d));
     }
     if (TEAM == 256) {
         const int wave = threadIdx.x >> 6;
@@ -583,6 +599,8 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
     case K_VEC64:
         quantize_vec<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds);
         break;
+    case K_VEC32: quantize_vec<T, 32>(s, p, blk * 8 + (tid >> 5), tid & 31, lds); break;
+    case K_VEC16: quantize_vec<T, 16>(s, p, blk * 16 + (tid >> 4), tid & 15, lds); break;
     case K_VEC8: quantize_vec<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
     case K_GEN64:
         quantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
@@ -704,6 +722,8 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
     case K_VEC64:
         dequantize_vec<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;
+    case K_VEC32: dequantize_vec<T, 32>(s, p, blk * 8 + (tid >> 5), tid & 31); break;
+    case K_VEC16: dequantize_vec<T, 16>(s, p, blk * 16 + (tid >> 4), tid & 15); break;
     case K_VEC8: dequantize_vec<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN64:
         dequantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
@@ -1014,20 +1034,23 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 // R_VPB 16-byte vectors per lane: R_VPB / UNITS peers of one row.  Loads carry
 // no branch: a lane past the end of the row re-reads the row's last vector, a
 // batch past the last peer re-reads the last peer, and both are ignored later.
-// Needs TEAM >= 64 (a peer's scale lives in one lane of each wavefront),
-// ws <= 64 and rows of at least one 16-byte vector.
+// Needs ws <= min(TEAM, 64) (lane l of a team, or of each of its wavefronts,
+// holds the scale of peer l) and rows of at least one 16-byte vector.  Teams
+// smaller than a wavefront take one row each; a team whose row is past the end
+// (`valid` false) works on the last row and stores nothing, so that the
+// wavefront stays converged for the cross-lane operations.
 constexpr int R_VPB = 4;
 
 template <int TEAM, int UNITS, bool PIPE, bool GDIV>
-DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane, float *lds)
+DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane, float *lds, bool valid = true)
 {
     constexpr int PB = R_VPB / UNITS >= 1 ? R_VPB / UNITS : 1;  // peers per batch
-    if (nrows <= 0) return;
+    if (TEAM >= 64 && nrows <= 0) return;
     const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
     const int ws = p.ws;
     const int nb = (ws + PB - 1) / PB;  // batches per row
     const int total = nrows * nb;
-    const int wlane = threadIdx.x & 63;
+    const int wlane = TEAM >= 64 ? (int)(threadIdx.x & 63u) : lane;
     const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
 
     // Vector u of this lane starts at dword doff[u].  The last vector of a row whose
@@ -1087,7 +1110,7 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
             for (int b = 0; b < PB; b++) {
                 const int k = cbatch * PB + b;
                 if (k < ws) {
-                    const float pr = bcast_lane(cr, k), pl = bcast_lane(cl, k);
+                    const float pr = team_bcast<TEAM>(cr, k), pl = team_bcast<TEAM>(cl, k);
 #pragma unroll
                     for (int u = 0; u < UNITS; u++) {
                         u32x4 w = src.w[b][u];
@@ -1112,10 +1135,10 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
 #pragma unroll
                 for (int u = 0; u < UNITS; u++) {
                     const u32x4 o = requant16<GDIV>(acc[u], s2, p);
-                    if (4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
+                    if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
                 }
-                if (lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
-            } else {
+                if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+            } else if (valid) {
                 reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
             }
 #pragma unroll
@@ -1234,7 +1257,24 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         }
         break;
     }
-    case K_GEN8: reduce_row<8, 1, GDIV>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
+    case K_GEN32:
+    case K_GEN16:
+    case K_GEN8: {
+        // one row per team of 32, 16 or 8 lanes
+        auto small = [&](auto team_c) {
+            constexpr int TEAM = decltype(team_c)::value;
+            const int j = blk * (TFTQ_WG / TEAM) + tid / TEAM;
+            if (p.ws <= TEAM) {
+                reduce_rows<TEAM, 1, true, GDIV>(s, p, min(j, s.slice_rows - 1), 1, tid % TEAM, lds, j < s.slice_rows);
+            } else {
+                reduce_row<TEAM, 1, GDIV>(s, p, j, tid % TEAM, lds);
+            }
+        };
+        if (s.kind[ST_R] == K_GEN32) small(std::integral_constant<int, 32>());
+        else if (s.kind[ST_R] == K_GEN16) small(std::integral_constant<int, 16>());
+        else small(std::integral_constant<int, 8>());
+        break;
+    }
     case K_GEN1: reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds); break;
     case K_COL1: reduce_col1<GDIV>(s, p, blk * 4 * TFTQ_WG, tid); break;
     default: break;

@@ -62,7 +62,11 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     const bool vec_ok = s.ptr != 0 && s.col_stride == 1 && in_bytes >= 64;
     if (s.n == 1 && s.ptr != 0) return K_COL1;
     if (vec_ok) {
+        // 8 vectors of 16 bytes per lane where the row is long enough, so that every
+        // lane has 8 loads in flight
         if (in_bytes <= 1024) return K_VEC8;
+        if (in_bytes <= 2048) return K_VEC16;
+        if (in_bytes <= 4096) return K_VEC32;
         if (in_bytes <= 8192) return K_VEC64;
         return K_VEC256;  // longer than 32 KB: two passes inside the workgroup
     }
@@ -78,6 +82,8 @@ static uint8_t pick_reduce_kind(const Seg &s)
     if (s.n == 1) return K_COL1;
     if (ndw <= 4) return K_GEN1;
     if (ndw <= 32) return K_GEN8;
+    if (ndw <= 64) return K_GEN16;
+    if (ndw <= 128) return K_GEN32;
     if (ndw <= 512) return K_GEN64;
     return K_GEN256;
 }
