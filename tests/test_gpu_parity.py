@@ -285,6 +285,36 @@ def test_short_rows_all_team_sizes(q, oracle, ws, op):
     full_check(q, oracle, half, ws, op, [ws // 2])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("ws", [1, 2, 8, 16])
+def test_short_rows_of_whole_vectors(q, oracle, dtype, ws):
+    """Contiguous rows of 1 ... 32 whole 16-byte vectors (8 ... 256 16-bit columns, 4 ... 128
+    fp32 columns): 1 to 8 lanes per row, several rows per lane; with rows past the end of
+    the tensor, padding rows, zero rows, rows that need the plain divide, a row stride larger
+    than the row and a base address that is only element-aligned."""
+    g = torch.Generator().manual_seed(7 * ws)
+    epv = 4 if dtype == torch.float32 else 8
+    vecs = [1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 24, 31, 32]
+    rows = [1, 7, 300, 1030, 2049]
+    peers = []
+    for p in range(ws):
+        ts = []
+        for i, nv in enumerate(vecs):
+            r, c = rows[i % len(rows)], nv * epv
+            x = torch.randn(r, c, generator=g) * (0.5 + p)
+            if r > 4:
+                x[1] *= 1e-30
+                x[2] = 0.0
+                x[3, 0] = -0.0
+            ts.append(x.to(dtype))
+        # row stride larger than the row, base one element off a 16-byte boundary
+        wide = (torch.randn(50 * 40 + 1, generator=g)).to(dtype)[1:].view(50, 40)[:, :2 * epv]
+        ts.append(wide)
+        peers.append(ts)
+    ranks = None if ws <= 2 else [0, ws - 1]
+    full_check(q, oracle, peers, ws, ReduceOp.AVG if ws % 2 else ReduceOp.SUM, ranks)
+
+
 def test_long_rows(q, oracle):
     """Rows longer than the register-resident paths hold: 20000 and 70000 columns."""
     g = torch.Generator().manual_seed(21)

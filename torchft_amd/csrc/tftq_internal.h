@@ -26,6 +26,7 @@ enum : uint8_t {
     K_GEN32 = 10,  // 32 lanes per row (reduce only)
     K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
     K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
+    K_VECS = 13,   // contiguous rows of at most 32 whole vectors: 1 to 8 lanes per row, several rows per lane
 };
 
 static inline int tftq_team_of(uint8_t kind)
@@ -42,6 +43,32 @@ static inline int tftq_team_of(uint8_t kind)
 }
 
 constexpr int TFTQ_WG = 256;       // threads per workgroup, all kernels
+
+// Helpers shared by the planner (host compiler) and the kernels (hipcc).
+#ifdef __HIPCC__
+#define TFTQ_HD __host__ __device__
+#else
+#define TFTQ_HD
+#endif
+
+// K_VECS: a row of nvec (1..32) 16-byte vectors is owned by a team of 2^lt lanes
+// (1, 2, 4 or 8), every lane holds 2^lc (1, 2 or 4) vectors of it, and works on
+// 8 >> lc rows at once, so that it has 8 loads in flight whatever the row length.
+TFTQ_HD static inline void tftq_small_shape(int nvec, int *lt, int *lc)
+{
+    int t = 0, c = 0;
+    while (t < 3 && (1 << t) < nvec) t++;
+    const int per_lane = (nvec + (1 << t) - 1) >> t;
+    while ((1 << c) < per_lane) c++;
+    *lt = t;
+    *lc = c;
+}
+static inline int tftq_small_rows_per_wg(int nvec)
+{
+    int lt, lc;
+    tftq_small_shape(nvec, &lt, &lc);
+    return (TFTQ_WG >> lt) * (8 >> lc);
+}
 constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
 
 // One tensor of the list.  64 bytes.

@@ -585,6 +585,89 @@ DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
     }
 }
 
+// Short contiguous rows of whole 16-byte vectors (K_VECS; the shape is
+// tftq_small_shape): 1 to 8 lanes per row, and every lane works on several rows
+// so that it has 8 loads in flight.  Row slot r of team t is row
+// row0 + r * teams + t: for a given r the teams of a wavefront read
+// consecutive rows, i.e. consecutive memory.
+struct SmallShape {
+    int lt, lc, team, teams, nrow, t, l;
+};
+DEV SmallShape small_shape(int nvec, int tid)
+{
+    SmallShape h;
+    tftq_small_shape(nvec, &h.lt, &h.lc);
+    h.team = 1 << h.lt;
+    h.teams = TFTQ_WG >> h.lt;
+    h.nrow = 8 >> h.lc;
+    h.t = tid >> h.lt;
+    h.l = tid & (h.team - 1);
+    return h;
+}
+
+// row -> byte offset of the packed row, with the slot found by one multiply
+// (inv = 1.0f / slice_rows; the estimate is off by at most one)
+DEV int64_t row_addr_fast(const Seg &s, int64_t slot_size, int row, float inv)
+{
+    int slot = (int)((float)row * inv);
+    int j = row - slot * s.slice_rows;
+    if (j < 0) { --slot; j += s.slice_rows; }
+    if (j >= s.slice_rows) { ++slot; j -= s.slice_rows; }
+    return (int64_t)slot * slot_size + s.slot_off + (int64_t)j * s.row_bytes;
+}
+
+template <typename T, int LC>
+DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int C = 1 << LC, ROWS = 8 >> LC;  // vectors per lane and row, rows per lane
+    const int nvec = s.n / EPV;
+    const int row0 = blk * (h.teams * ROWS);
+    const int m_pad = s.slice_rows * p.ws;
+    const float inv = 1.0f / (float)s.slice_rows;
+
+    u32x4 v[ROWS][C];
+    int row[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        row[r] = row0 + r * h.teams + h.t;
+        const int64_t e0 = (int64_t)min(row[r], s.m - 1) * s.row_stride;  // s.m >= 1: there are rows
+        GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + e0 * Elem<T>::ESZ);
+#pragma unroll
+        for (int k = 0; k < C; k++) v[r][k] = LOAD_STREAM(in + min(k * h.team + h.l, nvec - 1));
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        float a = 0.0f;
+#pragma unroll
+        for (int k = 0; k < C; k++) a = fmaxf(a, vec_absmax<T>(v[r][k]));
+        if (h.lt >= 1) a = fmaxf(a, dpp_mov<0xB1>(a));   // quad_perm [1,0,3,2]
+        if (h.lt >= 2) a = fmaxf(a, dpp_mov<0x4E>(a));   // quad_perm [2,3,0,1]
+        if (h.lt >= 3) a = fmaxf(a, dpp_mov<0x141>(a));  // row_half_mirror
+        if (row[r] >= m_pad) continue;
+        GLOBAL u32 *out = as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row[r], inv));
+        if (row[r] >= s.m) {
+            // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
+            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) out[d] = 0;
+            continue;
+        }
+        const float sc = calc_scale(a);
+        if (h.l == 0) out[0] = as_u(sc);
+#pragma unroll
+        for (int k = 0; k < C; k++)
+            if (k * h.team + h.l < nvec) vec_quant_store<T>(v[r][k], sc, out + 1, k * h.team + h.l);
+    }
+}
+
+template <typename T>
+DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid)
+{
+    const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
+    if (h.lc == 0) quantize_small_c<T, 0>(s, p, blk, tid, h);
+    else if (h.lc == 1) quantize_small_c<T, 1>(s, p, blk, tid, h);
+    else quantize_small_c<T, 2>(s, p, blk, tid, h);
+}
+
 template <typename T, bool INLINE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
@@ -608,6 +691,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
     case K_GEN8: quantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: quantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
     case K_COL1: quantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid); break;
+    case K_VECS: quantize_small<T>(s, p, blk, tid); break;
     default: break;
     }
 }
@@ -615,6 +699,17 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
 // ---------------------------------------------------------------------------
 // dequantize
 // ---------------------------------------------------------------------------
+// Streaming (nontemporal) stores pay off only when the pieces a store instruction
+// writes are whole 64-byte blocks: partial blocks written that way are not
+// merged in L2 (2000-byte bf16 rows: 3.5 TB/s streaming, 4.2 TB/s plain; 8000-byte
+// rows: 5.4 against 5.0).  True when the rows of the tensor start and end on
+// 64-byte boundaries.
+template <typename T>
+DEV bool rows_fill_lines(const Seg &s)
+{
+    return ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ) | (uint64_t)((int64_t)s.n * Elem<T>::ESZ)) & 63u) == 0;
+}
+
 // Any strides; also the path of rows whose scale is outside the range of the
 // fast exact division (plain IEEE divide, one element per lane and step).
 template <typename T, int TEAM>
@@ -642,8 +737,8 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
 // Contiguous, 16-byte aligned rows.  Four vectors per lane and step; their loads
 // are issued together without a branch (lanes past the end re-read the last
 // vector and do not store).
-template <typename T, int TEAM>
-DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
+template <typename T, int TEAM, bool NT>
+DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
 {
     if (row >= s.m) return;
     GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
@@ -686,9 +781,20 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
 #pragma unroll
                 for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(f[e], c.r, c.r_lo);
             }
-            if (idx < nvec) STORE_STREAM(Elem<T>::pack(o), out + idx);
+            if (idx < nvec) {
+                if (NT) STORE_STREAM(Elem<T>::pack(o), out + idx);
+                else out[idx] = Elem<T>::pack(o);
+            }
         }
     }
+}
+
+template <typename T, int TEAM>
+DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
+{
+    // same branch for the whole workgroup
+    if (rows_fill_lines<T>(s)) dequantize_vec_nt<T, TEAM, true>(s, p, row, lane);
+    else dequantize_vec_nt<T, TEAM, false>(s, p, row, lane);
 }
 
 // Rows of one column: one plain divide per row, four rows per lane.
@@ -706,6 +812,89 @@ DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
         const int row = row0 + k * TFTQ_WG + tid;
         const float f = __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0);
         if (row < s.m) Elem<T>::store(s.ptr, (int64_t)row * s.row_stride, f / as_f(w[k].x));  // no zero guard (:239)
+    }
+}
+
+// K_VECS in dequantize: same shape as quantize_small, 8 vectors of codes and their
+// rows' scales in flight per lane.
+template <typename T, int LC, bool NT>
+DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int C = 1 << LC, ROWS = 8 >> LC;
+    const int nvec = s.n / EPV;
+    const int row0 = blk * (h.teams * ROWS);
+    const float inv = 1.0f / (float)s.slice_rows;
+
+    u32x2 w[ROWS][C];
+    float sc[ROWS];
+    int row[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        row[r] = row0 + r * h.teams + h.t;
+        GLOBAL const u32 *in =
+            as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, min(row[r], s.m - 1), inv));
+        sc[r] = as_f(in[0]);
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            const int idx = min(k * h.team + h.l, nvec - 1);
+            if constexpr (EPV == 4) {
+                w[r][k].x = LOAD_STREAM(in + 1 + idx);
+                w[r][k].y = 0;
+            } else {
+                w[r][k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
+            }
+        }
+    }
+    bool all_fast = true;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) all_fast = all_fast && scale_is_fast(sc[r]);
+    const bool fast = __builtin_amdgcn_ballot_w64(!all_fast) == 0;  // one code path per wavefront
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const DivCoef c = make_div(sc[r]);
+        GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)min(row[r], s.m - 1) * s.row_stride * Elem<T>::ESZ);
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            float f[4], g[4], o[EPV];
+            unpack_fp8x4(w[r][k].x, f);
+            unpack_fp8x4(w[r][k].y, g);
+            if (fast) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], c.r, c.r_lo);
+                if constexpr (EPV == 8) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(g[e], c.r, c.r_lo);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = f[e] / sc[r];  // :250-252
+                if constexpr (EPV == 8) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[4 + e] = g[e] / sc[r];
+                }
+            }
+            const int vec = k * h.team + h.l;
+            if (row[r] < s.m && vec < nvec) {
+                if (NT) STORE_STREAM(Elem<T>::pack(o), out + vec);
+                else out[vec] = Elem<T>::pack(o);
+            }
+        }
+    }
+}
+
+template <typename T>
+DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid)
+{
+    const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
+    if (rows_fill_lines<T>(s)) {
+        if (h.lc == 0) dequantize_small_c<T, 0, true>(s, p, blk, tid, h);
+        else if (h.lc == 1) dequantize_small_c<T, 1, true>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 2, true>(s, p, blk, tid, h);
+    } else {
+        if (h.lc == 0) dequantize_small_c<T, 0, false>(s, p, blk, tid, h);
+        else if (h.lc == 1) dequantize_small_c<T, 1, false>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 2, false>(s, p, blk, tid, h);
     }
 }
 
@@ -733,6 +922,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
     case K_COL1:
         if (s.m > 0) dequantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid);
         break;
+    case K_VECS: dequantize_small<T>(s, p, blk, tid); break;
     default: break;
     }
 }

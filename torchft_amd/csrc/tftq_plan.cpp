@@ -61,6 +61,9 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     const int64_t in_bytes = (int64_t)s.n * esz;
     const bool vec_ok = s.ptr != 0 && s.col_stride == 1 && in_bytes >= 64;
     if (s.n == 1 && s.ptr != 0) return K_COL1;
+    const int epv = 16 / esz;
+    if (s.ptr != 0 && s.col_stride == 1 && s.n % epv == 0 && s.n / epv >= 1 && s.n / epv <= 32)
+        return K_VECS;  // short rows of whole vectors
     if (vec_ok) {
         // 8 vectors of 16 bytes per lane where the row is long enough, so that every
         // lane has 8 loads in flight
@@ -95,9 +98,10 @@ static uint8_t pick_reduce_kind(const Seg &s)
 // more loads in flight than one team's pipeline does.
 static int pick_reduce_rows(const Seg &, int) { return 1; }
 
-static int rows_per_wg_of(const Seg &s, int st)
+static int rows_per_wg_of(const Seg &s, int st, int esz)
 {
     if (s.kind[st] == K_COL1) return 4 * TFTQ_WG;
+    if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
     const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
     return st == ST_R ? teams * s.reduce_rows_per_team : teams;
 }
@@ -105,7 +109,7 @@ static int rows_per_wg_of(const Seg &s, int st)
 // Bytes one workgroup of segment s moves in a stage.
 static double wg_weight(const Seg &s, int st, int esz, int ws)
 {
-    const double rows = (double)rows_per_wg_of(s, st);
+    const double rows = (double)rows_per_wg_of(s, st, esz);
     if (st == ST_R) return rows * (double)s.row_bytes * (ws + 1);
     return rows * ((double)s.n * esz + (double)s.row_bytes);
 }
@@ -281,7 +285,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         s.reduce_rows_per_team = (uint8_t)pick_reduce_rows(s, ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
-            const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st));
+            const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st, p->esz));
             wgs[i][st] = (int32_t)n;
             wg[st] += n;
             if (wg[st] > INT32_MAX - 4096) {
