@@ -1465,7 +1465,11 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         else small(std::integral_constant<int, 8>());
         break;
     }
-    case K_GEN1: reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds); break;
+    case K_GEN1:  // one lane per row: 1, 2 or 4 vectors of codes per peer
+        if (ndw <= 4) reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        else if (ndw <= 8) reduce_row<1, 2, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        else reduce_row<1, 4, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        break;
     case K_COL1: reduce_col1<GDIV>(s, p, blk * 4 * TFTQ_WG, tid); break;
     default: break;
     }

@@ -83,7 +83,7 @@ static uint8_t pick_reduce_kind(const Seg &s)
     // one or two 16-byte vectors of codes per lane and peer, four for the longest rows
     const int ndw = s.row_bytes / 4 - 1;
     if (s.n == 1) return K_COL1;
-    if (ndw <= 4) return K_GEN1;
+    if (ndw <= 16) return K_GEN1;  // up to 64 bytes of codes: a lane per row beats a team with idle lanes
     if (ndw <= 32) return K_GEN8;
     if (ndw <= 64) return K_GEN16;
     if (ndw <= 128) return K_GEN32;
