@@ -45,10 +45,15 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--sets", type=int, default=3, help="buffer sets the steps rotate over")
     ap.add_argument("--rank", type=int, default=None)
-    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat"],
+    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat", "shape"],
                     help="workload: 3 = Llama-3-8B layer bucket (the headline, default); 2, 4, 5 = the "
                          "other GPU configurations; flat = one 1-D fp32 tensor of 64 Mi elements "
-                         "(what a bucketised DiLoCo all-reduce passes)")
+                         "(what a bucketised DiLoCo all-reduce passes); shape = --shape")
+    ap.add_argument("--shape", default="53248x4096",
+                    help="with --config shape: ROWSxCOLS[,ROWSxCOLS...], N(0, 0.02) values")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16", "float32"],
+                    help="with --config shape")
+    ap.add_argument("--ws", type=int, default=8, help="with --config shape: group size (reduce AVG)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a counter "
@@ -150,6 +155,16 @@ def main() -> int:
                                            generator=torch.Generator(device=dev).manual_seed(seed))],
                  8, ReduceOp.SUM, "one 1-D fp32 tensor of 67108864 elements (rows of one column), ws=8, SUM"),
     }
+    if args.config == "shape":
+        shapes = [tuple(int(d) for d in part.split("x")) for part in args.shape.split(",")]
+        dt = getattr(torch, args.dtype)
+
+        def make_shape(seed):
+            g = torch.Generator(device=dev).manual_seed(seed)
+            return [(torch.randn(sh, device=dev, generator=g) * 0.02).to(dt) for sh in shapes]
+
+        table["shape"] = (make_shape, args.ws, ReduceOp.AVG,
+                          f"tensors {args.shape} {args.dtype}, N(0, 0.02), ws={args.ws}, AVG")
     make, ws, op, workload_name = table[args.config]
     rank = args.rank if args.rank is not None else min(3, ws - 1)
     if args.config == "4":
@@ -276,7 +291,7 @@ def main() -> int:
     # The roofline entry is for the kernel that takes the largest share of the step.
     # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE (x2.000,
     # calibrated on a 256 MiB copy) + WRITE_SIZE (x1.000); profiles/cfg3_bf16_ws8_hbm_traffic.md
-    measured_traffic = {"quantize": 654942000, "reduce": 247438000, "dequantize": 660774000}
+    measured_traffic = {"quantize": 654952000, "reduce": 247230000, "dequantize": 661279000}
     achieved = ab[dominant] / (dominant_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "k_" + dominant, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
