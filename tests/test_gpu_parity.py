@@ -508,3 +508,75 @@ def test_wrapper_errors_on_gpu(q):
         q.fused_dequantize_from_fp8(x, buf[:-4], 2)
     with pytest.raises(RuntimeError):
         q.fused_reduce_fp8(x, buf, 2, 2)
+
+
+@pytest.mark.parametrize("n_tensors", [3, 20])
+def test_entry_points_under_graph_capture(q, n_tensors):
+    """The three entry points only enqueue kernels on the stream they are given, so a HIP
+    graph can capture them.  The graph is replayed several times with new inputs and with
+    eager work and synchronisations in between; every replay must equal the eager result."""
+    from torchft_amd import _lib
+    L = _lib.load()
+    ws, rank = 4, 2
+    g = torch.Generator().manual_seed(77)
+    shapes = [(37, 4096), (50, 333), (1900, 1), (64, 64), (9, 1000)]
+    ts = [torch.randn(shapes[i % len(shapes)], generator=g).to(torch.bfloat16).cuda() for i in range(n_tensors)]
+    outs = [torch.empty_like(t) for t in ts]
+    T = len(ts)
+
+    def plan_for(tensors):
+        ptrs = (ctypes.c_void_p * T)(*[t.data_ptr() for t in tensors])
+        sh = (ctypes.c_int64 * (2 * T))(*[v for t in tensors for v in t.shape])
+        st = (ctypes.c_int64 * (2 * T))(*[v for t in tensors for v in t.stride()])
+        h = ctypes.c_void_p()
+        assert L.tftq_plan_create(2, T, ptrs, sh, st, ws, ctypes.byref(h)) == 0
+        table = None
+        nbytes = L.tftq_plan_table_bytes(h)
+        if nbytes:
+            host = (ctypes.c_uint8 * nbytes).from_address(L.tftq_plan_table_host(h))
+            table = torch.frombuffer(host, dtype=torch.uint8).cuda()
+            assert L.tftq_plan_set_device_table(h, ctypes.c_void_p(table.data_ptr())) == 0
+        return h, table
+
+    h_in, keep_in = plan_for(ts)     # quantize and reduce read `ts`
+    h_out, keep_out = plan_for(outs)  # dequantize writes `outs`
+    size = L.tftq_plan_output_size(h_in)
+    packed = torch.empty(size, dtype=torch.uint8, device="cuda")
+
+    def enqueue(stream):
+        s = ctypes.c_void_p(stream.cuda_stream)
+        p = ctypes.c_void_p(packed.data_ptr())
+        assert L.tftq_quantize(h_in, p, size, s) == 0
+        assert L.tftq_reduce(h_in, p, size, rank, 1, s) == 0
+        assert L.tftq_dequantize(h_out, p, size, s) == 0
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue(side)  # warm-up outside the capture
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            enqueue(torch.cuda.current_stream())
+    torch.cuda.current_stream().wait_stream(side)
+
+    for it in range(4):
+        for t in ts:
+            t.copy_((torch.randn(t.shape, generator=g) * (it + 1)).to(torch.bfloat16))
+        for o in outs:
+            o.zero_()
+        packed.fill_(0x5A)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        got_packed = packed.clone()
+        for o in outs:
+            o.zero_()
+        packed.fill_(0x5A)
+        enqueue(torch.cuda.current_stream())  # eager, same inputs
+        torch.cuda.synchronize()
+        same_bytes(got_packed, packed, f"replay {it}: packed buffer")
+        for i, (a, b) in enumerate(zip(got, outs)):
+            same_bytes(a, b, f"replay {it}: tensor {i}")
+    L.tftq_plan_destroy(h_in)
+    L.tftq_plan_destroy(h_out)
