@@ -315,6 +315,22 @@ def test_short_rows_of_whole_vectors(q, oracle, dtype, ws):
     full_check(q, oracle, peers, ws, ReduceOp.AVG if ws % 2 else ReduceOp.SUM, ranks)
 
 
+def test_wide_rows(q, oracle):
+    """Rows between the regular and the doubled register capacity (16-bit inputs: 16392 to
+    32768 columns) run in the kernel variants with more registers, alone and next to short rows."""
+    g = torch.Generator().manual_seed(23)
+    # 32772 / 32776 / 32780 columns: two passes in chunks of 1024 dwords with 1, 2, 3 dwords left
+    # over, whose last vector reaches back into codes that were already replaced in place
+    for dtype, cols in ((torch.bfloat16, [16392, 28672, 32768, 32772, 32776, 32780]),
+                        (torch.float32, [8200, 16384, 20000, 36868])):
+        peers = [[torch.randn(3, c, generator=g).to(dtype) * (p + 1) for c in cols] +
+                 [torch.randn(70, 512, generator=g).to(dtype)] for p in range(4)]
+        for t in peers[1]:
+            t[1] *= 1e-30  # the exact fallback
+        full_check(q, oracle, peers, 4, ReduceOp.AVG)
+        full_check(q, oracle, peers[:3], 3, ReduceOp.AVG, ranks=[2])
+
+
 def test_long_rows(q, oracle):
     """Rows longer than the register-resident paths hold: 20000 and 70000 columns."""
     g = torch.Generator().manual_seed(21)

@@ -71,6 +71,14 @@ static inline int tftq_small_rows_per_wg(int nvec)
 }
 constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
 
+// Rows a workgroup can hold in registers.  The regular kernels keep up to 8
+// input vectors per lane in quantize (rows of 2048 vectors = 32 KB) and the
+// accumulators of 4096 payload dwords (16384 columns) in reduce; the "wide"
+// kernel variants hold twice that at half the occupancy and are launched only
+// for plans that contain such rows.  Longer rows make two passes.
+constexpr int TFTQ_Q_VECS = 8 * TFTQ_WG, TFTQ_Q_VECS_WIDE = 16 * TFTQ_WG;
+constexpr int TFTQ_R_DWORDS = 4096, TFTQ_R_DWORDS_WIDE = 8192;
+
 // One tensor of the list.  64 bytes.
 struct Seg {
     uint64_t ptr;        // device address of element (0,0); 0 for reduce-only plans
@@ -132,6 +140,7 @@ struct tftq_plan {
     int64_t output_size;
     int64_t max_rows;
     int32_t nwg[3];
+    bool wide[3];              // per stage: some row needs the kernel variant with more registers
     Dealt dealt[3];            // inline table only
     int32_t dealt_per_xcd[3];  // inline table only: workgroups of the busiest XCD
     TableIndex index[3];       // device table only

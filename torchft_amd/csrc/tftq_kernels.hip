@@ -439,6 +439,10 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     amax = team_max<TEAM>(amax, lds);
     const float sc = calc_scale(amax);
     if (lane == 0) out[0] = as_u(sc);
+    // The elements are unpacked again from the raw vectors: keeping the floats of the
+    // maximum search alive until here would double the registers of 16-bit inputs.
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) asm volatile("" : "+v"(v[k].x), "+v"(v[k].y), "+v"(v[k].z), "+v"(v[k].w));
 #pragma unroll
     for (int k = 0; k < KMAX; k++) {
         const int idx = k * TEAM + lane;
@@ -511,12 +515,14 @@ DEV void quantize_vec_long(const Seg &s, const KParams &p, int row, int tid, flo
     }
 }
 
-template <typename T, int TEAM>
+template <typename T, int TEAM, bool WIDE>
 DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds)
 {
     // same branch for the whole workgroup
-    if (s.n / Elem<T>::EPV <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
-    else if (TEAM < 256 || s.n / Elem<T>::EPV <= QV * TEAM) quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
+    const int nvec = s.n / Elem<T>::EPV;
+    if (nvec <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
+    else if (TEAM < 256 || nvec <= TFTQ_Q_VECS) quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
+    else if (WIDE && nvec <= TFTQ_Q_VECS_WIDE) quantize_vec_k<T, TEAM, 2 * QV>(s, p, row, lane, lds);
     else quantize_vec_long<T>(s, p, row, lane, lds);
 }
 
@@ -668,7 +674,7 @@ DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid)
     else quantize_small_c<T, 2>(s, p, blk, tid, h);
 }
 
-template <typename T, bool INLINE>
+template <typename T, bool INLINE, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
@@ -678,13 +684,13 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
     const int blk = vb - s.wg_begin[ST_Q];
     const int tid = threadIdx.x;
     switch (s.kind[ST_Q]) {
-    case K_VEC256: quantize_vec<T, 256>(s, p, blk, tid, lds); break;
+    case K_VEC256: quantize_vec<T, 256, WIDE>(s, p, blk, tid, lds); break;
     case K_VEC64:
-        quantize_vec<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds);
+        quantize_vec<T, 64, false>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds);
         break;
-    case K_VEC32: quantize_vec<T, 32>(s, p, blk * 8 + (tid >> 5), tid & 31, lds); break;
-    case K_VEC16: quantize_vec<T, 16>(s, p, blk * 16 + (tid >> 4), tid & 15, lds); break;
-    case K_VEC8: quantize_vec<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
+    case K_VEC32: quantize_vec<T, 32, false>(s, p, blk * 8 + (tid >> 5), tid & 31, lds); break;
+    case K_VEC16: quantize_vec<T, 16, false>(s, p, blk * 16 + (tid >> 4), tid & 15, lds); break;
+    case K_VEC8: quantize_vec<T, 8, false>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
     case K_GEN64:
         quantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;
@@ -1107,7 +1113,19 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
                 // the moved-back last vector overlaps its neighbour, which may sit in another
                 // wavefront: nobody stores before everybody has read the own slot's chunk
                 __syncthreads();
-                if (valid) *(GLOBAL u32x4_a4 *)(orow + 1 + doff) = requant16<GDIV>(acc, s2, p);
+                if (valid) {
+                    const u32x4 o = requant16<GDIV>(acc, s2, p);
+                    if (doff >= d) {
+                        *(GLOBAL u32x4_a4 *)(orow + 1 + doff) = o;
+                    } else {
+                        // The vector reaches back into the previous chunk, whose codes have
+                        // already been replaced in the own slot: what was accumulated for
+                        // those dwords is meaningless and they are final already.
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (doff + e >= d) orow[1 + doff + e] = o[e];
+                    }
+                }
             }
         }
         if (pass == 0) {
@@ -1398,7 +1416,7 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
     }
 }
 
-template <bool INLINE, bool GDIV>
+template <bool INLINE, bool GDIV, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
@@ -1413,7 +1431,9 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
     case K_GEN256: {
         const int j0 = blk * rpt;
         const int nrows = min(rpt, s.slice_rows - j0);
-        if (ndw > 4096) {
+        if (WIDE && ndw > TFTQ_R_DWORDS && ndw <= TFTQ_R_DWORDS_WIDE && p.ws <= 64) {
+            reduce_rows<256, 8, false, GDIV>(s, p, j0, nrows, tid, lds);
+        } else if (ndw > TFTQ_R_DWORDS) {
             for (int r = 0; r < nrows; r++) {
                 if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
                 else reduce_row_long<GDIV>(s, p, j0 + r, tid, lds);
@@ -1538,12 +1558,16 @@ static inline unsigned grid_of(const KParams &kp)
 }
 
 template <typename T>
-static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, hipStream_t st)
+static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, hipStream_t st)
 {
-    if (use_inline)
-        hipLaunchKernelGGL((k_quantize<T, true>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
-    else
-        hipLaunchKernelGGL((k_quantize<T, false>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
+    const dim3 grid(grid_of(kp)), block(TFTQ_WG);
+    if (wide) {
+        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, true>), grid, block, 0, st, kp, inl);
+        else hipLaunchKernelGGL((k_quantize<T, false, true>), grid, block, 0, st, kp, inl);
+    } else {
+        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, false>), grid, block, 0, st, kp, inl);
+        else hipLaunchKernelGGL((k_quantize<T, false, false>), grid, block, 0, st, kp, inl);
+    }
     return (int)hipGetLastError();
 }
 
@@ -1570,9 +1594,9 @@ extern "C" int tftq_quantize(const tftq_plan *plan, void *packed, int64_t packed
     if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
     switch (plan->dtype) {
-    case TFTQ_F32: return launch_q<float>(kp, inl, use_inline, st);
-    case TFTQ_F16: return launch_q<f16_tag>(kp, inl, use_inline, st);
-    case TFTQ_BF16: return launch_q<bf16_tag>(kp, inl, use_inline, st);
+    case TFTQ_F32: return launch_q<float>(kp, inl, use_inline, plan->wide[ST_Q], st);
+    case TFTQ_F16: return launch_q<f16_tag>(kp, inl, use_inline, plan->wide[ST_Q], st);
+    case TFTQ_BF16: return launch_q<bf16_tag>(kp, inl, use_inline, plan->wide[ST_Q], st);
     default: return TFTQ_E_DTYPE;
     }
 }
@@ -1621,12 +1645,15 @@ extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_b
     if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid(grid_of(kp)), block(TFTQ_WG);
-    if (kp.div_mode == 2) {
-        if (use_inline) hipLaunchKernelGGL((k_reduce<true, true>), grid, block, 0, st, kp, inl);
-        else hipLaunchKernelGGL((k_reduce<false, true>), grid, block, 0, st, kp, inl);
+    const bool gdiv = kp.div_mode == 2;
+#define TFTQ_LAUNCH_R(I, G, W) hipLaunchKernelGGL((k_reduce<I, G, W>), grid, block, 0, st, kp, inl)
+    if (plan->wide[ST_R]) {
+        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, true); else TFTQ_LAUNCH_R(false, true, true); }
+        else { if (use_inline) TFTQ_LAUNCH_R(true, false, true); else TFTQ_LAUNCH_R(false, false, true); }
     } else {
-        if (use_inline) hipLaunchKernelGGL((k_reduce<true, false>), grid, block, 0, st, kp, inl);
-        else hipLaunchKernelGGL((k_reduce<false, false>), grid, block, 0, st, kp, inl);
+        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, false); else TFTQ_LAUNCH_R(false, true, false); }
+        else { if (use_inline) TFTQ_LAUNCH_R(true, false, false); else TFTQ_LAUNCH_R(false, false, false); }
     }
+#undef TFTQ_LAUNCH_R
     return (int)hipGetLastError();
 }
