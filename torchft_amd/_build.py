@@ -5,17 +5,19 @@ from __future__ import annotations
 import os
 import shutil
 import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libtftq.so")
-SOURCES = ["tftq_kernels.hip", "tftq_plan.cpp"]
+SOURCES = ["tftq_quantize.hip", "tftq_reduce.hip", "tftq_dequantize.hip", "tftq_plan.cpp"]
 
 # -ffp-contract=off: the arithmetic contract is separate IEEE multiply, divide
 # and add; fused multiply-adds are written out where they are wanted.
 # packed-fp32-ops off: no v_pk_*_f32 instructions are generated.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
@@ -29,15 +31,26 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found; libtftq.so cannot be built")
 
 
-def build_library(verbose: bool = False) -> str:
-    """Compile unconditionally and return the path of the shared library."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", LIB_PATH,
-           *[os.path.join(CSRC, s) for s in SOURCES]]
+def _run(cmd: list[str]) -> str:
     res = subprocess.run(cmd, cwd=CSRC, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines()
                     if "packed-fp32-ops" not in l)  # host pass does not know the feature
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
+    return out
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile unconditionally and return the path of the shared library.  The
+    sources are compiled side by side (one hipcc per file), then linked."""
+    hipcc = hipcc_path()
+    with tempfile.TemporaryDirectory(prefix="tftq_build_") as tmp:
+        objs = [os.path.join(tmp, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+        cmds = [[hipcc, *HIPCC_FLAGS, "-c", "-o", o, os.path.join(CSRC, s)] for s, o in zip(SOURCES, objs)]
+        with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
+            outs = list(pool.map(_run, cmds))
+        outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]))
+    out = "\n".join(o for o in outs if o.strip())
     if verbose and out.strip():
         print(out)
     return LIB_PATH

@@ -1,0 +1,267 @@
+// k_dequantize and tftq_dequantize: fused_dequantize_from_fp8 on gfx950.
+//
+// Follows torchft/quantization.py:165-258 (kernel) and :591-635 (launcher); design notes in tftq_device.h.
+
+#include "tftq_device.h"
+
+// ---------------------------------------------------------------------------
+// dequantize
+// ---------------------------------------------------------------------------
+// Streaming (nontemporal) stores pay off only when the pieces a store instruction
+// writes are whole 64-byte blocks: partial blocks written that way are not
+// merged in L2 (2000-byte bf16 rows: 3.5 TB/s streaming, 4.2 TB/s plain; 8000-byte
+// rows: 5.4 against 5.0).  True when the rows of the tensor start and end on
+// 64-byte boundaries.
+template <typename T>
+DEV bool rows_fill_lines(const Seg &s)
+{
+    return ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ) | (uint64_t)((int64_t)s.n * Elem<T>::ESZ)) & 63u) == 0;
+}
+
+// Any strides; also the path of rows whose scale is outside the range of the
+// fast exact division (plain IEEE divide, one element per lane and step).
+template <typename T, int TEAM>
+DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
+{
+    if (row >= s.m) return;
+    GLOBAL const uint8_t *in = as_global<const uint8_t>(p.packed + row_addr(s, p.slot_size, row));
+    const DivCoef c = make_div(as_f(*(GLOBAL const u32 *)in));  // no zero guard (:239)
+    const uint64_t base = s.ptr;
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    if (c.fast) {
+        for (int col = lane; col < s.n; col += TEAM) {
+            const float f = __builtin_amdgcn_cvt_f32_fp8((int)in[4 + col], 0);
+            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, div_fast_signed(f, c.r, c.r_lo));
+        }
+    } else {
+#pragma nounroll
+        for (int col = lane; col < s.n; col += TEAM) {
+            const float f = __builtin_amdgcn_cvt_f32_fp8((int)in[4 + col], 0);
+            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, f / c.s);
+        }
+    }
+}
+
+// Contiguous, 16-byte aligned rows.  Four vectors per lane and step; their loads
+// are issued together without a branch (lanes past the end re-read the last
+// vector and do not store).
+template <typename T, int TEAM, bool NT>
+DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
+{
+    if (row >= s.m) return;
+    GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
+    const DivCoef c = make_div(as_f(in[0]));
+    if (!c.fast) {  // same for all lanes of the team
+        dequantize_gen<T, TEAM>(s, p, row, lane);
+        return;
+    }
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int DV = 8;  // loads in flight per lane (4: 1.3 % slower on 4096-column bf16 rows)
+    const int nvec = s.n / EPV;
+    GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
+    // the few columns after the last whole vector, one element per lane
+    for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
+        const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
+        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, div_fast_signed(f, c.r, c.r_lo));
+    }
+    for (int base = 0; base < nvec; base += DV * TEAM) {
+        u32x2 w[DV];
+#pragma unroll
+        for (int k = 0; k < DV; k++) {
+            const int idx = min(base + k * TEAM + lane, nvec - 1);
+            if constexpr (EPV == 4) {
+                w[k].x = LOAD_STREAM(in + 1 + idx);
+                w[k].y = 0;
+            } else {
+                w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < DV; k++) {
+            const int idx = base + k * TEAM + lane;
+            float o[EPV];
+            float f[4];
+            unpack_fp8x4(w[k].x, f);
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], c.r, c.r_lo);
+            if constexpr (EPV == 8) {
+                unpack_fp8x4(w[k].y, f);
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(f[e], c.r, c.r_lo);
+            }
+            if (idx < nvec) {
+                if (NT) STORE_STREAM(Elem<T>::pack(o), out + idx);
+                else out[idx] = Elem<T>::pack(o);
+            }
+        }
+    }
+}
+
+template <typename T, int TEAM>
+DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
+{
+    // same branch for the whole workgroup
+    if (rows_fill_lines<T>(s)) dequantize_vec_nt<T, TEAM, true>(s, p, row, lane);
+    else dequantize_vec_nt<T, TEAM, false>(s, p, row, lane);
+}
+
+// Rows of one column: one plain divide per row, four rows per lane.
+template <typename T>
+DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+{
+    u32x2 w[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = min(row0 + k * TFTQ_WG + tid, s.m - 1);
+        w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)as_global<const u32>(p.packed + row_addr(s, p.slot_size, row)));
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = row0 + k * TFTQ_WG + tid;
+        const float f = __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0);
+        if (row < s.m) Elem<T>::store(s.ptr, (int64_t)row * s.row_stride, f / as_f(w[k].x));  // no zero guard (:239)
+    }
+}
+
+// K_VECS in dequantize: same shape as quantize_small, 8 vectors of codes and their
+// rows' scales in flight per lane.
+template <typename T, int LC, bool NT>
+DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int C = 1 << LC, ROWS = 8 >> LC;
+    const int nvec = s.n / EPV;
+    const int row0 = blk * (h.teams * ROWS);
+    const float inv = 1.0f / (float)s.slice_rows;
+
+    u32x2 w[ROWS][C];
+    float sc[ROWS];
+    int row[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        row[r] = row0 + r * h.teams + h.t;
+        GLOBAL const u32 *in =
+            as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, min(row[r], s.m - 1), inv));
+        sc[r] = as_f(in[0]);
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            const int idx = min(k * h.team + h.l, nvec - 1);
+            if constexpr (EPV == 4) {
+                w[r][k].x = LOAD_STREAM(in + 1 + idx);
+                w[r][k].y = 0;
+            } else {
+                w[r][k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
+            }
+        }
+    }
+    bool all_fast = true;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) all_fast = all_fast && scale_is_fast(sc[r]);
+    const bool fast = __builtin_amdgcn_ballot_w64(!all_fast) == 0;  // one code path per wavefront
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const DivCoef c = make_div(sc[r]);
+        GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)min(row[r], s.m - 1) * s.row_stride * Elem<T>::ESZ);
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            float f[4], g[4], o[EPV];
+            unpack_fp8x4(w[r][k].x, f);
+            unpack_fp8x4(w[r][k].y, g);
+            if (fast) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], c.r, c.r_lo);
+                if constexpr (EPV == 8) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(g[e], c.r, c.r_lo);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = f[e] / sc[r];  // :250-252
+                if constexpr (EPV == 8) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[4 + e] = g[e] / sc[r];
+                }
+            }
+            const int vec = k * h.team + h.l;
+            if (row[r] < s.m && vec < nvec) {
+                if (NT) STORE_STREAM(Elem<T>::pack(o), out + vec);
+                else out[vec] = Elem<T>::pack(o);
+            }
+        }
+    }
+}
+
+template <typename T>
+DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid)
+{
+    const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
+    if (rows_fill_lines<T>(s)) {
+        if (h.lc == 0) dequantize_small_c<T, 0, true>(s, p, blk, tid, h);
+        else if (h.lc == 1) dequantize_small_c<T, 1, true>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 2, true>(s, p, blk, tid, h);
+    } else {
+        if (h.lc == 0) dequantize_small_c<T, 0, false>(s, p, blk, tid, h);
+        else if (h.lc == 1) dequantize_small_c<T, 1, false>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 2, false>(s, p, blk, tid, h);
+    }
+}
+
+template <typename T, bool INLINE>
+__global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const InlineTable inl)
+{
+    Seg s;
+    int vb;
+    if (!locate<INLINE, ST_D>(p, inl, s, vb)) return;
+    const int blk = vb - s.wg_begin[ST_D];
+    const int tid = threadIdx.x;
+    switch (s.kind[ST_D]) {
+    case K_VEC256: dequantize_vec<T, 256>(s, p, blk, tid); break;
+    case K_VEC64:
+        dequantize_vec<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
+        break;
+    case K_VEC32: dequantize_vec<T, 32>(s, p, blk * 8 + (tid >> 5), tid & 31); break;
+    case K_VEC16: dequantize_vec<T, 16>(s, p, blk * 16 + (tid >> 4), tid & 15); break;
+    case K_VEC8: dequantize_vec<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
+    case K_GEN64:
+        dequantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
+        break;
+    case K_GEN8: dequantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
+    case K_GEN1: dequantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
+    case K_COL1:
+        if (s.m > 0) dequantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid);
+        break;
+    case K_VECS: dequantize_small<T>(s, p, blk, tid); break;
+    default: break;
+    }
+}
+
+template <typename T>
+static int launch_d(const KParams &kp, const InlineTable &inl, bool use_inline, hipStream_t st)
+{
+    if (use_inline)
+        hipLaunchKernelGGL((k_dequantize<T, true>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
+    else
+        hipLaunchKernelGGL((k_dequantize<T, false>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
+    return (int)hipGetLastError();
+}
+
+extern "C" int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
+                               void *stream)
+{
+    KParams kp;
+    InlineTable inl = {};
+    bool use_inline;
+    int rc = fill_params(plan, ST_D, (void *)packed, packed_bytes, &kp, &inl, &use_inline);
+    if (rc) return rc;
+    for (int i = 0; i < plan->nseg; i++)
+        if (plan->segs[(size_t)i].ptr == 0 && plan->segs[(size_t)i].m > 0 && plan->segs[(size_t)i].n > 0)
+            return TFTQ_E_ARG;
+    if (kp.nwg == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    switch (plan->dtype) {
+    case TFTQ_F32: return launch_d<float>(kp, inl, use_inline, st);
+    case TFTQ_F16: return launch_d<f16_tag>(kp, inl, use_inline, st);
+    case TFTQ_BF16: return launch_d<bf16_tag>(kp, inl, use_inline, st);
+    default: return TFTQ_E_DTYPE;
+    }
+}

@@ -1,5 +1,5 @@
 // Shared between the host-side planner (tftq_plan.cpp) and the HIP kernels
-// (tftq_kernels.hip).  Not part of the public ABI.
+// (tftq_device.h and the three .hip files).  Not part of the public ABI.
 #pragma once
 
 #include <stdint.h>

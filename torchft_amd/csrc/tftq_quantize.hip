@@ -1,0 +1,341 @@
+// k_quantize and tftq_quantize: fused_quantize_into_fp8 on gfx950.
+//
+// Follows torchft/quantization.py:53-162 (kernel) and :531-588 (launcher); design notes in tftq_device.h.
+
+#include "tftq_device.h"
+
+// ---------------------------------------------------------------------------
+// quantize
+// ---------------------------------------------------------------------------
+constexpr int QV = 8;  // 16-byte vectors a lane keeps in registers
+
+template <typename T>
+DEV float vec_absmax(const u32x4 v)
+{
+    float f[Elem<T>::EPV];
+    Elem<T>::unpack(v, f);
+    float a = 0.0f;
+#pragma unroll
+    for (int e = 0; e < Elem<T>::EPV; e++) a = fmaxf(a, __builtin_fabsf(f[e]));
+    return a;
+}
+
+template <typename T>
+DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
+{
+    float f[Elem<T>::EPV];
+    Elem<T>::unpack(v, f);
+    if constexpr (Elem<T>::EPV == 4) {
+        payload[idx] = pack_fp8x4(f[0] * s, f[1] * s, f[2] * s, f[3] * s);
+    } else {
+        u32x2 o;
+        o.x = pack_fp8x4(f[0] * s, f[1] * s, f[2] * s, f[3] * s);
+        o.y = pack_fp8x4(f[4] * s, f[5] * s, f[6] * s, f[7] * s);
+        *(GLOBAL u32x2_a4 *)(payload + 2 * idx) = o;  // plain store: rows start 4 bytes off a line, L2 merges
+    }
+}
+
+// Contiguous, 16-byte aligned rows of at most TEAM * KMAX vectors.  The KMAX
+// loads of a lane are issued back to back without a branch in between: lanes
+// past the end of the row re-read its last vector (a duplicate cannot change
+// the maximum) and simply do not store.
+template <typename T, int TEAM, int KMAX>
+DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float *lds)
+{
+    const bool active = row < s.slice_rows * p.ws;
+    GLOBAL u32 *out = as_global<u32>(p.packed + (active ? row_addr(s, p.slot_size, row) : 0));
+    if (active && row >= s.m) {
+        // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
+        for (int d = lane; d < (s.row_bytes >> 2); d += TEAM) out[d] = 0;
+    }
+    if (!active || row >= s.m) return;  // a team leaves whole: its lanes share the row
+
+    constexpr int EPV = Elem<T>::EPV;
+    const int nvec = s.n / EPV;
+    const int tail = s.n - nvec * EPV;  // elements after the last whole vector (rare)
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
+    u32x4 v[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) v[k] = LOAD_STREAM(in + min(k * TEAM + lane, nvec - 1));
+    float t[EPV - 1];
+    if (tail) {  // every lane reads the few tail elements; lane 0 will store their codes
+#pragma unroll
+        for (int e = 0; e < EPV - 1; e++) t[e] = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(e, tail - 1));
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+    if (tail) {
+#pragma unroll
+        for (int e = 0; e < EPV - 1; e++) amax = fmaxf(amax, __builtin_fabsf(t[e]));
+    }
+    amax = team_max<TEAM>(amax, lds);
+    const float sc = calc_scale(amax);
+    if (lane == 0) out[0] = as_u(sc);
+    // The elements are unpacked again from the raw vectors: keeping the floats of the
+    // maximum search alive until here would double the registers of 16-bit inputs.
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) asm volatile("" : "+v"(v[k].x), "+v"(v[k].y), "+v"(v[k].z), "+v"(v[k].w));
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) {
+        const int idx = k * TEAM + lane;
+        if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
+    }
+    if (tail && lane == 0) {
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) y[e] = (e < EPV - 1 && e < tail) ? t[e < EPV - 1 ? e : 0] * sc : 0.0f;
+        GLOBAL u32 *tw = out + 1 + nvec * (EPV / 4);
+        u32 w0 = pack_fp8x4(y[0], y[1], y[2], y[3]);
+        if (tail < 4) w0 &= (1u << (8 * tail)) - 1u;  // padding bytes are zero whatever 0 * sc gave
+        tw[0] = w0;
+        if (EPV == 8 && tail > 4) {
+            u32 w1 = pack_fp8x4(y[4], y[5], y[6], y[7]);
+            if (tail < 8) w1 &= (1u << (8 * (tail - 4))) - 1u;
+            tw[1] = w1;
+        }
+    }
+}
+
+// Rows of more than 32 KB: too long for the registers of a workgroup.  Two
+// passes with 16-byte loads; the second one finds the row in the caches.
+template <typename T>
+DEV void quantize_vec_long(const Seg &s, const KParams &p, int row, int tid, float *lds)
+{
+    const bool active = row < s.slice_rows * p.ws;
+    if (!active) return;
+    GLOBAL u32 *out = as_global<u32>(p.packed + row_addr(s, p.slot_size, row));
+    if (row >= s.m) {
+        for (int d = tid; d < (s.row_bytes >> 2); d += TFTQ_WG) out[d] = 0;
+        return;
+    }
+    constexpr int EPV = Elem<T>::EPV;
+    const int nvec = s.n / EPV;
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
+    float amax = 0.0f;
+    for (int c = nvec * EPV + tid; c < s.n; c += TFTQ_WG) amax = fmaxf(amax, __builtin_fabsf(Elem<T>::load(s.ptr, r0 + c)));
+#pragma nounroll
+    for (int base = 0; base < nvec; base += 4 * TFTQ_WG) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = in[min(base + k * TFTQ_WG + tid, nvec - 1)];
+#pragma unroll
+        for (int k = 0; k < 4; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+    }
+    amax = team_max<256>(amax, lds);
+    const float sc = calc_scale(amax);
+    if (tid == 0) out[0] = as_u(sc);
+#pragma nounroll
+    for (int base = 0; base < nvec; base += 4 * TFTQ_WG) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = LOAD_STREAM(in + min(base + k * TFTQ_WG + tid, nvec - 1));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int idx = base + k * TFTQ_WG + tid;
+            if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
+        }
+    }
+    // tail: at most EPV - 1 elements after the last whole vector, byte stores plus zero padding
+    if (tid == 0) {
+        const int c0 = nvec * EPV;
+        GLOBAL uint8_t *ob = (GLOBAL uint8_t *)(out + 1);
+        for (int c = c0; c < ((s.n + 3) & ~3); c++) {
+            const float x = c < s.n ? Elem<T>::load(s.ptr, r0 + c) : 0.0f;
+            ob[c] = c < s.n ? (uint8_t)(pack_fp8x4(x * sc, 0.0f, 0.0f, 0.0f) & 0xFFu) : (uint8_t)0;
+        }
+    }
+}
+
+template <typename T, int TEAM, bool WIDE>
+DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds)
+{
+    // same branch for the whole workgroup
+    const int nvec = s.n / Elem<T>::EPV;
+    if (nvec <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
+    else if (TEAM < 256 || nvec <= TFTQ_Q_VECS) quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
+    else if (WIDE && nvec <= TFTQ_Q_VECS_WIDE) quantize_vec_k<T, TEAM, 2 * QV>(s, p, row, lane, lds);
+    else quantize_vec_long<T>(s, p, row, lane, lds);
+}
+
+// Any strides, any alignment, any n: element loads, two passes over the row
+// (the second one is served by the caches).
+template <typename T, int TEAM>
+DEV void quantize_gen(const Seg &s, const KParams &p, int row, int lane)
+{
+    const bool active = row < s.slice_rows * p.ws;
+    if (!active) return;
+    GLOBAL u32 *out = as_global<u32>(p.packed + row_addr(s, p.slot_size, row));
+    const int ndw = (s.row_bytes >> 2) - 1;
+    if (row >= s.m) {
+        for (int d = lane; d <= ndw; d += TEAM) out[d] = 0;
+        return;
+    }
+    const uint64_t base = s.ptr;
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    float amax = 0.0f;
+    for (int c = lane; c < s.n; c += TEAM)
+        amax = fmaxf(amax, __builtin_fabsf(Elem<T>::load(base, r0 + (int64_t)c * s.col_stride)));
+    amax = team_max<TEAM>(amax, nullptr);
+    const float sc = calc_scale(amax);
+    if (lane == 0) out[0] = as_u(sc);
+    for (int d = lane; d < ndw; d += TEAM) {
+        float y[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int c = 4 * d + e;
+            const float x = c < s.n ? Elem<T>::load(base, r0 + (int64_t)c * s.col_stride) : 0.0f;
+            y[e] = x * sc;
+        }
+        u32 w = pack_fp8x4(y[0], y[1], y[2], y[3]);
+        const int tail = s.n - 4 * d;  // codes of this dword that belong to the row
+        if (tail < 4) w &= (1u << (8 * tail)) - 1u;  // zero padding, whatever 0 * sc gave
+        out[1 + d] = w;
+    }
+}
+
+// Rows of one column (1-D tensors, quantization.py:487-488): a row is its own
+// maximum, so the code is +-448 (or 0) and all information is in the scale.
+// Four rows per lane, interleaved so that every load and every 8-byte
+// [scale, code] store of a wavefront is contiguous.
+template <typename T>
+DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+{
+    const int m_pad = s.slice_rows * p.ws;
+    float x[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = min(row0 + k * TFTQ_WG + tid, s.m - 1);
+        x[k] = s.m > 0 ? Elem<T>::load(s.ptr, (int64_t)row * s.row_stride) : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int row = row0 + k * TFTQ_WG + tid;
+        if (row < m_pad) {
+            u32x2 o = {0u, 0u};  // padding rows stay zero
+            if (row < s.m) {
+                const float sc = calc_scale(__builtin_fabsf(x[k]));
+                o.x = as_u(sc);
+                o.y = pack_fp8x4(x[k] * sc, 0.0f, 0.0f, 0.0f) & 0xFFu;
+            }
+            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + row_addr(s, p.slot_size, row)) = o;
+        }
+    }
+}
+
+// Short contiguous rows of whole 16-byte vectors (K_VECS, shape in tftq_device.h).
+template <typename T, int LC>
+DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int C = 1 << LC, ROWS = 8 >> LC;  // vectors per lane and row, rows per lane
+    const int nvec = s.n / EPV;
+    const int row0 = blk * (h.teams * ROWS);
+    const int m_pad = s.slice_rows * p.ws;
+    const float inv = 1.0f / (float)s.slice_rows;
+
+    u32x4 v[ROWS][C];
+    int row[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        row[r] = row0 + r * h.teams + h.t;
+        const int64_t e0 = (int64_t)min(row[r], s.m - 1) * s.row_stride;  // s.m >= 1: there are rows
+        GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + e0 * Elem<T>::ESZ);
+#pragma unroll
+        for (int k = 0; k < C; k++) v[r][k] = LOAD_STREAM(in + min(k * h.team + h.l, nvec - 1));
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        float a = 0.0f;
+#pragma unroll
+        for (int k = 0; k < C; k++) a = fmaxf(a, vec_absmax<T>(v[r][k]));
+        if (h.lt >= 1) a = fmaxf(a, dpp_mov<0xB1>(a));   // quad_perm [1,0,3,2]
+        if (h.lt >= 2) a = fmaxf(a, dpp_mov<0x4E>(a));   // quad_perm [2,3,0,1]
+        if (h.lt >= 3) a = fmaxf(a, dpp_mov<0x141>(a));  // row_half_mirror
+        if (row[r] >= m_pad) continue;
+        GLOBAL u32 *out = as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row[r], inv));
+        if (row[r] >= s.m) {
+            // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
+            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) out[d] = 0;
+            continue;
+        }
+        const float sc = calc_scale(a);
+        if (h.l == 0) out[0] = as_u(sc);
+#pragma unroll
+        for (int k = 0; k < C; k++)
+            if (k * h.team + h.l < nvec) vec_quant_store<T>(v[r][k], sc, out + 1, k * h.team + h.l);
+    }
+}
+
+template <typename T>
+DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid)
+{
+    const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
+    if (h.lc == 0) quantize_small_c<T, 0>(s, p, blk, tid, h);
+    else if (h.lc == 1) quantize_small_c<T, 1>(s, p, blk, tid, h);
+    else quantize_small_c<T, 2>(s, p, blk, tid, h);
+}
+
+template <typename T, bool INLINE, bool WIDE>
+__global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
+{
+    __shared__ float lds[4];
+    Seg s;
+    int vb;
+    if (!locate<INLINE, ST_Q>(p, inl, s, vb)) return;
+    const int blk = vb - s.wg_begin[ST_Q];
+    const int tid = threadIdx.x;
+    switch (s.kind[ST_Q]) {
+    case K_VEC256: quantize_vec<T, 256, WIDE>(s, p, blk, tid, lds); break;
+    case K_VEC64:
+        quantize_vec<T, 64, false>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds);
+        break;
+    case K_VEC32: quantize_vec<T, 32, false>(s, p, blk * 8 + (tid >> 5), tid & 31, lds); break;
+    case K_VEC16: quantize_vec<T, 16, false>(s, p, blk * 16 + (tid >> 4), tid & 15, lds); break;
+    case K_VEC8: quantize_vec<T, 8, false>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
+    case K_GEN64:
+        quantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
+        break;
+    case K_GEN8: quantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
+    case K_GEN1: quantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
+    case K_COL1: quantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid); break;
+    case K_VECS: quantize_small<T>(s, p, blk, tid); break;
+    default: break;
+    }
+}
+
+template <typename T>
+static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, hipStream_t st)
+{
+    const dim3 grid(grid_of(kp)), block(TFTQ_WG);
+    if (wide) {
+        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, true>), grid, block, 0, st, kp, inl);
+        else hipLaunchKernelGGL((k_quantize<T, false, true>), grid, block, 0, st, kp, inl);
+    } else {
+        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, false>), grid, block, 0, st, kp, inl);
+        else hipLaunchKernelGGL((k_quantize<T, false, false>), grid, block, 0, st, kp, inl);
+    }
+    return (int)hipGetLastError();
+}
+
+extern "C" int tftq_quantize(const tftq_plan *plan, void *packed, int64_t packed_bytes, void *stream)
+{
+    KParams kp;
+    InlineTable inl = {};
+    bool use_inline;
+    int rc = fill_params(plan, ST_Q, packed, packed_bytes, &kp, &inl, &use_inline);
+    if (rc) return rc;
+    for (int i = 0; i < plan->nseg; i++)
+        if (plan->segs[(size_t)i].ptr == 0 && plan->segs[(size_t)i].m > 0 && plan->segs[(size_t)i].n > 0)
+            return TFTQ_E_ARG;
+    if (kp.nwg == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    switch (plan->dtype) {
+    case TFTQ_F32: return launch_q<float>(kp, inl, use_inline, plan->wide[ST_Q], st);
+    case TFTQ_F16: return launch_q<f16_tag>(kp, inl, use_inline, plan->wide[ST_Q], st);
+    case TFTQ_BF16: return launch_q<bf16_tag>(kp, inl, use_inline, plan->wide[ST_Q], st);
+    default: return TFTQ_E_DTYPE;
+    }
+}

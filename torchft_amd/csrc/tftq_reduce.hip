@@ -1,0 +1,620 @@
+// k_reduce, tftq_reduce and tftq_check_device: fused_reduce_fp8 on gfx950.
+//
+// Follows torchft/quantization.py:261-428 (kernels) and :638-686 (launcher); design notes in tftq_device.h.
+
+#include "tftq_device.h"
+
+// ---------------------------------------------------------------------------
+// reduce
+// ---------------------------------------------------------------------------
+// Loads dwords [d0, d0+4) of a row payload (ndw dwords long); dwords past the
+// end read as 0 and are never touched in memory.  Codes past column n inside
+// the last dword are cleared: the reference masks them (:420-424).
+DEV u32x4 load_codes(GLOBAL const u32 *payload, int d0, int ndw, int n)
+{
+    u32x4 w = {0, 0, 0, 0};
+    const int rem = ndw - d0;
+    if (rem >= 4) {
+        w = *(GLOBAL const u32x4_a4 *)(payload + d0);
+    } else if (rem > 0) {
+        w.x = payload[d0];
+        if (rem > 1) w.y = payload[d0 + 1];
+        if (rem > 2) w.z = payload[d0 + 2];
+    }
+    if (n & 3) {
+        const int last = ndw - 1 - d0;
+        const u32 mask = (1u << (8 * (n & 3))) - 1u;
+        if (last == 0) w.x &= mask;
+        if (last == 1) w.y &= mask;
+        if (last == 2) w.z &= mask;
+        if (last == 3) w.w &= mask;
+    }
+    return w;
+}
+
+DEV void store_codes(GLOBAL u32 *payload, int d0, int ndw, const u32x4 w)
+{
+    const int rem = ndw - d0;
+    if (rem >= 4) {
+        *(GLOBAL u32x4_a4 *)(payload + d0) = w;
+    } else if (rem > 0) {
+        payload[d0] = w.x;
+        if (rem > 1) payload[d0 + 1] = w.y;
+        if (rem > 2) payload[d0 + 2] = w.z;
+    }
+}
+
+// acc[e] += code[e] / s for the 16 codes of w, s given as (r, r_lo)
+DEV void accumulate16(float (&acc)[16], const u32x4 w, float r, float r_lo)
+{
+    const u32 ww[4] = {w.x, w.y, w.z, w.w};
+
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        float f[4];
+        unpack_fp8x4(ww[t], f);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[4 * t + e] = acc[4 * t + e] + div_fast(f[e], r, r_lo);
+    }
+}
+
+// (acc * s2) / div, left to right (:364).  GDIV: div is not a power of two
+// and needs a real divide; otherwise inv_div (1 for SUM) is an exact inverse
+// and multiplying by it is the same correctly rounded result.
+template <bool GDIV>
+DEV float scale_div(float a, float s2, const KParams &p)
+{
+    const float y = a * s2;
+    return GDIV ? y / p.div : y * p.inv_div;
+}
+
+template <bool GDIV>
+DEV u32x4 requant16(const float (&a)[16], float s2, const KParams &p)
+{
+    float y[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) y[e] = scale_div<GDIV>(a[e], s2, p);
+    u32x4 o;
+    o.x = pack_fp8x4(y[0], y[1], y[2], y[3]);
+    o.y = pack_fp8x4(y[4], y[5], y[6], y[7]);
+    o.z = pack_fp8x4(y[8], y[9], y[10], y[11]);
+    o.w = pack_fp8x4(y[12], y[13], y[14], y[15]);
+    return o;
+}
+
+DEV GLOBAL const u32 *peer_row(const KParams &p, int k, int64_t off)
+{
+    int peer = p.rank + k;  // :407
+    if (peer >= p.ws) peer -= p.ws;
+
+    return as_global<const u32>(p.packed + (int64_t)peer * p.slot_size + off);
+}
+
+DEV float guarded_scale(GLOBAL const u32 *prow)
+{
+    const float sc = as_f(prow[0]);
+    return sc == 0.0f ? 1.0f : sc;  // padding rows (:419)
+}
+
+// One column at a time with plain IEEE divides, two passes: the path of rows
+// in which some peer's scale is outside the range of the fast exact division,
+// and of rows too long for registers.  Small code, not tuned.
+template <int TEAM, bool GDIV>
+DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float *lds)
+{
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    GLOBAL uint8_t *orow = as_global<uint8_t>(p.packed + (int64_t)p.rank * p.slot_size + off);
+    float amax = 0.0f, s2 = 0.0f;
+#pragma nounroll
+    for (int pass = 0; pass < 2; pass++) {
+#pragma nounroll
+        for (int c = lane; c < s.n; c += TEAM) {
+            float a = 0.0f;
+#pragma nounroll
+            for (int k = 0; k < p.ws; k++) {
+                GLOBAL const u32 *prow = peer_row(p, k, off);
+                const float sc = guarded_scale(prow);
+                const int code = ((GLOBAL const uint8_t *)prow)[4 + c];
+                a = a + __builtin_amdgcn_cvt_f32_fp8(code, 0) / sc;
+            }
+            if (pass == 0) {
+                amax = fmaxf(amax, __builtin_fabsf(a));
+            } else {
+                const float y = scale_div<GDIV>(a, s2, p);
+                orow[4 + c] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(y, 0.0f, 0, false) & 0xFF);
+            }
+        }
+        if (pass == 0) {
+            amax = team_max<TEAM>(amax, lds);
+            s2 = calc_scale(amax / p.div);
+        }
+    }
+    // the own slot's old scale is an input of every lane: write the new one last (:375)
+    __threadfence_block();
+    if (TEAM == 256) __syncthreads();
+    if (lane == 0) *(GLOBAL u32 *)orow = as_u(s2);
+}
+
+// Rows longer than a 256-lane team can keep in registers (more than 16384
+// columns): two passes over chunks of 1024 dwords, as the reference does for
+// every row (:318-372), but with 16-byte loads, the fast exact division and the
+// scales read once.  The second pass finds the peer rows in the caches.
+template <bool GDIV>
+DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *lds)
+{
+    const int ndw = (s.row_bytes >> 2) - 1;
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    const int wlane = tid & 63;
+    const int ws = p.ws;  // <= 64 here
+    const DivCoef c = make_div(guarded_scale(peer_row(p, min(wlane, ws - 1), off)));
+    if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // same in the four wavefronts
+        reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
+        return;
+    }
+    GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+    const u32 tailmask = (s.n & 3) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+    float amax = 0.0f, s2 = 0.0f;
+#pragma nounroll
+    for (int pass = 0; pass < 2; pass++) {
+#pragma nounroll
+        for (int d = 0; d < ndw; d += 4 * TFTQ_WG) {
+            const bool valid = d + 4 * tid < ndw;
+            const int doff = min(d + 4 * tid, ndw - 4);  // the last vector ends with the row
+            const u32 mask = doff == ndw - 4 ? tailmask : 0xFFFFFFFFu;
+            float acc[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+#pragma nounroll
+            for (int k0 = 0; k0 < ws; k0 += 4) {
+                u32x4 w[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k0 + b, ws - 1), off) + 1 + doff));
+                }
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    w[b].w &= mask;
+                    if (k0 + b < ws) accumulate16(acc, w[b], bcast_lane(c.r, k0 + b), bcast_lane(c.r_lo, k0 + b));
+                }
+            }
+            if (pass == 0) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[e]));
+            } else {
+                // the moved-back last vector overlaps its neighbour, which may sit in another
+                // wavefront: nobody stores before everybody has read the own slot's chunk
+                __syncthreads();
+                if (valid) {
+                    const u32x4 o = requant16<GDIV>(acc, s2, p);
+                    if (doff >= d) {
+                        *(GLOBAL u32x4_a4 *)(orow + 1 + doff) = o;
+                    } else {
+                        // The vector reaches back into the previous chunk, whose codes have
+                        // already been replaced in the own slot: what was accumulated for
+                        // those dwords is meaningless and they are final already.
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (doff + e >= d) orow[1 + doff + e] = o[e];
+                    }
+                }
+            }
+        }
+        if (pass == 0) {
+            amax = team_max<256>(amax, lds);  // every wavefront has read the old scales by now
+            s2 = calc_scale(amax / p.div);
+        }
+    }
+    if (tid == 0) orow[0] = as_u(s2);  // :375
+}
+
+// Register-resident row: the team holds all accumulators of the row, each peer
+// row is read once.  UNITS = 16-byte vectors of codes per lane and peer.
+template <int TEAM, int UNITS, bool GDIV>
+DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
+{
+    constexpr int PB = 8 / UNITS;  // peers whose loads are in flight together
+    if (j >= s.slice_rows) return;  // a team leaves whole: its lanes share the row
+    const int ndw = (s.row_bytes >> 2) - 1;
+    const int n = s.n;
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    const int wlane = threadIdx.x & 63;
+
+    float acc[UNITS][16];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+
+    for (int kc = 0; kc < p.ws; kc += 64) {
+        const int kend = min(p.ws, kc + 64);
+        // Wide teams: lane l of every wavefront fetches the scale of peer kc + l
+        // first, then the codes of the first peers go in flight, and only then
+        // are the scales turned into division coefficients.
+        float my_scale = 1.0f;
+        if (TEAM >= 64 && kc + wlane < p.ws) my_scale = guarded_scale(peer_row(p, kc + wlane, off));
+
+        u32x4 w[PB][UNITS];
+        float sraw[PB];
+        auto load_batch = [&](int k0) {
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                if (k0 + b < kend) {
+                    GLOBAL const u32 *prow = peer_row(p, k0 + b, off);
+                    if (TEAM < 64) sraw[b] = guarded_scale(prow);
+#pragma unroll
+                    for (int u = 0; u < UNITS; u++)
+                        w[b][u] = load_codes(prow + 1, (u * TEAM + lane) * 4, ndw, n);
+                }
+            }
+        };
+        load_batch(kc);
+
+        float cr = 1.0f, cl = 0.0f;
+        if (TEAM >= 64) {
+            const DivCoef c = make_div(my_scale);
+            cr = c.r;
+            cl = c.r_lo;
+            if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // some peer needs the plain divide
+                reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);
+                return;
+            }
+        }
+        for (int k0 = kc; k0 < kend; k0 += PB) {
+            if (k0 != kc) load_batch(k0);
+            if (TEAM < 64) {
+                bool fast = true;
+#pragma unroll
+                for (int b = 0; b < PB; b++)
+                    if (k0 + b < kend) fast = fast && scale_is_fast(sraw[b]);
+                if (!fast) {  // same decision in every lane of the team
+                    reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);
+                    return;
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                if (k0 + b < kend) {
+                    float pr, pl;
+                    if (TEAM >= 64) {
+                        pr = bcast_lane(cr, k0 + b - kc);
+                        pl = bcast_lane(cl, k0 + b - kc);
+                    } else {
+                        const DivCoef c = make_div(sraw[b]);
+                        pr = c.r;
+                        pl = c.r_lo;
+                    }
+#pragma unroll
+                    for (int u = 0; u < UNITS; u++) accumulate16(acc[u], w[b][u], pr, pl);
+                }
+            }
+        }
+    }
+
+    float amax = 0.0f;
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+    amax = team_max<TEAM>(amax, lds);
+    const float s2 = calc_scale(amax / p.div);  // :340
+
+    GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+        store_codes(orow + 1, (u * TEAM + lane) * 4, ndw, requant16<GDIV>(acc[u], s2, p));
+    // Every lane read the old scale of the own slot before team_max (wide
+    // teams synchronise there; narrow teams are one wavefront in program order).
+    if (lane == 0) orow[0] = as_u(s2);  // :375
+}
+
+// Several rows per team, software-pipelined: the codes of the next batch of
+// peers (of this row or of the next row) are in flight while the current batch
+// is accumulated, so a wavefront always has loads outstanding.  A batch is
+// R_VPB 16-byte vectors per lane: R_VPB / UNITS peers of one row.  Loads carry
+// no branch: a lane past the end of the row re-reads the row's last vector, a
+// batch past the last peer re-reads the last peer, and both are ignored later.
+// Needs ws <= min(TEAM, 64) (lane l of a team, or of each of its wavefronts,
+// holds the scale of peer l) and rows of at least one 16-byte vector.  Teams
+// smaller than a wavefront take one row each; a team whose row is past the end
+// (`valid` false) works on the last row and stores nothing, so that the
+// wavefront stays converged for the cross-lane operations.
+constexpr int R_VPB = 4;
+
+template <int TEAM, int UNITS, bool PIPE, bool GDIV>
+DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane, float *lds, bool valid = true)
+{
+    constexpr int PB = R_VPB / UNITS >= 1 ? R_VPB / UNITS : 1;  // peers per batch
+    if (TEAM >= 64 && nrows <= 0) return;
+    const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
+    const int ws = p.ws;
+    const int nb = (ws + PB - 1) / PB;  // batches per row
+    const int total = nrows * nb;
+    const int wlane = TEAM >= 64 ? (int)(threadIdx.x & 63u) : lane;
+    const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
+
+    // Vector u of this lane starts at dword doff[u].  The last vector of a row whose
+    // length is not a multiple of 4 dwords is moved back so that it ends with the row:
+    // it overlaps its neighbour, both lanes compute and store the same values.  Lanes
+    // past the row's end re-read the last vector and do not store.
+    int doff[UNITS];
+    u32 padmask[UNITS];  // clears the bytes past column n in the row's last dword (:420-424)
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        doff[u] = min(4 * (u * TEAM + lane), ndw - 4);
+        padmask[u] = (doff[u] == ndw - 4 && (s.n & 3)) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+    }
+
+    struct Batch {
+        u32x4 w[PB][UNITS];
+        float scale;  // lane l: guarded scale of peer min(l, ws-1) of the batch's row
+    };
+    Batch A, B;
+
+    int lrow = 0, lbatch = 0;  // next batch to load
+    auto issue = [&](Batch &dst) {
+        const int64_t off = s.slot_off + (int64_t)(j0 + lrow) * s.row_bytes;
+        dst.scale = as_f(peer_row(p, speer, off)[0]);
+#pragma unroll
+        for (int b = 0; b < PB; b++) {
+            GLOBAL const u32 *pv = peer_row(p, min(lbatch * PB + b, ws - 1), off) + 1;
+#pragma unroll
+            for (int u = 0; u < UNITS; u++)
+                dst.w[b][u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + doff[u]));
+        }
+        if (++lbatch == nb) {
+            lbatch = 0;
+            ++lrow;
+        }
+    };
+
+    float acc[UNITS][16];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+    int crow = 0, cbatch = 0;  // batch being consumed
+    float cr = 1.0f, cl = 0.0f;
+    bool row_fast = true;
+
+    auto consume = [&](const Batch &src) {
+        if (cbatch == 0) {
+            const float sc = src.scale == 0.0f ? 1.0f : src.scale;  // padding rows (:419)
+            const DivCoef c = make_div(sc);
+            cr = c.r;
+            cl = c.r_lo;
+            row_fast = __builtin_amdgcn_ballot_w64(!c.fast) == 0;  // same in all wavefronts of the team
+        }
+        if (row_fast) {
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                const int k = cbatch * PB + b;
+                if (k < ws) {
+                    const float pr = team_bcast<TEAM>(cr, k), pl = team_bcast<TEAM>(cl, k);
+#pragma unroll
+                    for (int u = 0; u < UNITS; u++) {
+                        u32x4 w = src.w[b][u];
+                        w.w &= padmask[u];  // here, not at the load: the load must stay in flight
+                        accumulate16(acc[u], w, pr, pl);
+                    }
+                }
+            }
+        }
+        if (++cbatch == nb) {
+            const int j = j0 + crow;
+            if (row_fast) {
+                float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
+#pragma unroll
+                for (int u = 0; u < UNITS; u++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+                amax = team_max<TEAM>(amax, lds);
+                const float s2 = calc_scale(amax / p.div);  // :340
+                const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+                GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+#pragma unroll
+                for (int u = 0; u < UNITS; u++) {
+                    const u32x4 o = requant16<GDIV>(acc[u], s2, p);
+                    if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
+                }
+                if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+            } else if (valid) {
+                reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
+            }
+#pragma unroll
+            for (int u = 0; u < UNITS; u++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+            cbatch = 0;
+            ++crow;
+        }
+    };
+
+    if (!PIPE) {  // long rows: one batch in flight keeps the register count down
+        for (int i = 0; i < total; i++) {
+            issue(A);
+            consume(A);
+        }
+        return;
+    }
+    issue(A);
+    int i = 0;
+    for (; i + 2 < total; i += 2) {
+        issue(B);
+        consume(A);
+        issue(A);
+        consume(B);
+    }
+    if (i + 1 < total) {
+        issue(B);
+        consume(A);
+        consume(B);
+    } else {
+        consume(A);
+    }
+}
+
+// Rows of one column: 8 bytes per row and peer, one plain divide per peer
+// (coefficients for the fast division would cost two), four rows per lane.
+template <bool GDIV>
+DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
+{
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    int64_t off[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        off[k] = s.slot_off + (int64_t)min(j0 + k * TFTQ_WG + tid, s.slice_rows - 1) * 8;
+#pragma nounroll
+    for (int kk = 0; kk < p.ws; kk++) {
+        u32x2 w[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)peer_row(p, kk, off[k]));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float sc = as_f(w[k].x);
+            sc = sc == 0.0f ? 1.0f : sc;  // padding rows (:419)
+            acc[k] = acc[k] + __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0) / sc;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        if (j0 + k * TFTQ_WG + tid < s.slice_rows) {
+            const float s2 = calc_scale(__builtin_fabsf(acc[k]) / p.div);
+            u32x2 o;
+            o.x = as_u(s2);
+            o.y = pack_fp8x4(scale_div<GDIV>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
+            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off[k]) = o;
+        }
+    }
+}
+
+template <bool INLINE, bool GDIV, bool WIDE>
+__global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
+{
+    __shared__ float lds[4];
+    Seg s;
+    int vb;
+    if (!locate<INLINE, ST_R>(p, inl, s, vb)) return;
+    const int blk = vb - s.wg_begin[ST_R];
+    const int tid = threadIdx.x;
+    const int ndw = (s.row_bytes >> 2) - 1;
+    const int rpt = s.reduce_rows_per_team;
+    switch (s.kind[ST_R]) {
+    case K_GEN256: {
+        const int j0 = blk * rpt;
+        const int nrows = min(rpt, s.slice_rows - j0);
+        if (WIDE && ndw > TFTQ_R_DWORDS && ndw <= TFTQ_R_DWORDS_WIDE && p.ws <= 64) {
+            reduce_rows<256, 8, false, GDIV>(s, p, j0, nrows, tid, lds);
+        } else if (ndw > TFTQ_R_DWORDS) {
+            for (int r = 0; r < nrows; r++) {
+                if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
+                else reduce_row_long<GDIV>(s, p, j0 + r, tid, lds);
+            }
+        } else if (p.ws > 64) {
+            for (int r = 0; r < nrows; r++) {
+                if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j0 + r, tid, lds);
+                else reduce_row<256, 4, GDIV>(s, p, j0 + r, tid, lds);
+            }
+        } else if (ndw <= 1024) {
+            reduce_rows<256, 1, true, GDIV>(s, p, j0, nrows, tid, lds);
+        } else if (ndw <= 2048) {
+            reduce_rows<256, 2, true, GDIV>(s, p, j0, nrows, tid, lds);
+        } else {
+            reduce_rows<256, 4, false, GDIV>(s, p, j0, nrows, tid, lds);
+        }
+        break;
+    }
+    case K_GEN64: {
+        const int j0 = (blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6)) * rpt;
+        const int nrows = min(rpt, s.slice_rows - j0);
+        if (p.ws > 64) {
+            for (int r = 0; r < nrows; r++) {
+                if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j0 + r, tid & 63, lds);
+                else reduce_row<64, 2, GDIV>(s, p, j0 + r, tid & 63, lds);
+            }
+        } else if (ndw <= 256) {
+            reduce_rows<64, 1, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
+        } else {
+            reduce_rows<64, 2, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
+        }
+        break;
+    }
+    case K_GEN32:
+    case K_GEN16:
+    case K_GEN8: {
+        // one row per team of 32, 16 or 8 lanes
+        auto small = [&](auto team_c) {
+            constexpr int TEAM = decltype(team_c)::value;
+            const int j = blk * (TFTQ_WG / TEAM) + tid / TEAM;
+            if (p.ws <= TEAM) {
+                reduce_rows<TEAM, 1, true, GDIV>(s, p, min(j, s.slice_rows - 1), 1, tid % TEAM, lds, j < s.slice_rows);
+            } else {
+                reduce_row<TEAM, 1, GDIV>(s, p, j, tid % TEAM, lds);
+            }
+        };
+        if (s.kind[ST_R] == K_GEN32) small(std::integral_constant<int, 32>());
+        else if (s.kind[ST_R] == K_GEN16) small(std::integral_constant<int, 16>());
+        else small(std::integral_constant<int, 8>());
+        break;
+    }
+    case K_GEN1:  // one lane per row: 1, 2 or 4 vectors of codes per peer
+        if (ndw <= 4) reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        else if (ndw <= 8) reduce_row<1, 2, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        else reduce_row<1, 4, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        break;
+    case K_COL1: reduce_col1<GDIV>(s, p, blk * 4 * TFTQ_WG, tid); break;
+    default: break;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+extern "C" int tftq_check_device(void)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return (int)e;
+    const char *a = prop.gcnArchName;
+    return (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')
+               ? 0
+               : TFTQ_E_ARCH;
+}
+
+extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank,
+                           int is_avg, void *stream)
+{
+    KParams kp;
+    InlineTable inl = {};
+    bool use_inline;
+    int rc = fill_params(plan, ST_R, packed, packed_bytes, &kp, &inl, &use_inline);
+    if (rc) return rc;
+    if (rank < 0 || rank >= plan->ws) return TFTQ_E_ARG;
+    kp.rank = rank;
+    if (is_avg) {
+        const int ws = plan->ws;
+        kp.div = (float)ws;
+        if ((ws & (ws - 1)) == 0) {
+            kp.div_mode = 1;
+            kp.inv_div = 1.0f / (float)ws;
+        } else {
+            kp.div_mode = 2;
+        }
+    }
+    if (kp.nwg == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(grid_of(kp)), block(TFTQ_WG);
+    const bool gdiv = kp.div_mode == 2;
+#define TFTQ_LAUNCH_R(I, G, W) hipLaunchKernelGGL((k_reduce<I, G, W>), grid, block, 0, st, kp, inl)
+    if (plan->wide[ST_R]) {
+        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, true); else TFTQ_LAUNCH_R(false, true, true); }
+        else { if (use_inline) TFTQ_LAUNCH_R(true, false, true); else TFTQ_LAUNCH_R(false, false, true); }
+    } else {
+        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, false); else TFTQ_LAUNCH_R(false, true, false); }
+        else { if (use_inline) TFTQ_LAUNCH_R(true, false, false); else TFTQ_LAUNCH_R(false, false, false); }
+    }
+#undef TFTQ_LAUNCH_R
+    return (int)hipGetLastError();
+}
