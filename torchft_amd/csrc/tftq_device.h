@@ -8,16 +8,18 @@
 //   k_dequantize<T>  fused_dequantize_from_fp8 (:165-258)
 //
 // Design (none of it follows the reference's launch shape):
-//   * a row is owned by a "team" of 1, 8, 64 or 256 lanes chosen from the row
-//     length; the team loads the row once with 16-byte loads, keeps it in
+//   * a row is owned by a "team" of 1 to 256 lanes chosen from the row length
+//     (so that a lane has about 8 loads of 16 bytes in flight; lanes of very
+//     short rows work on several rows); the team loads the row once, keeps it in
 //     registers, reduces |x| with DPP inside the wavefront (LDS across the four
 //     wavefronts of a 256-lane team) and converts from registers with the
 //     packed fp8 converts of gfx950.  Every stage reads HBM once.
 //   * all tensors of a call are covered by one launch: a workgroup finds its
 //     tensor in a table of 64-byte descriptors (in the kernel arguments for
 //     short lists) and branches on the team size stored there.
-//   * workgroup ids are remapped so that each of the 8 XCDs works on one
-//     contiguous range of rows (neighbouring packed rows share cache lines).
+//   * workgroup ids are remapped so that each of the 8 XCDs works on
+//     contiguous pieces of every tensor (neighbouring packed rows share cache
+//     lines), in reduce the tensors with the heaviest workgroups first.
 //   * division by a row scale is exact IEEE division, computed as
 //     fma(f, r, f * r_lo) with r = RN(1/s) and r_lo = RN(fma(-s, r, 1) / s).
 //     For the 253 finite e4m3 values f and every binary32 s with exponent in
