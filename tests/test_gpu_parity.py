@@ -596,3 +596,48 @@ def test_entry_points_under_graph_capture(q, n_tensors):
             same_bytes(a, b, f"replay {it}: tensor {i}")
     L.tftq_plan_destroy(h_in)
     L.tftq_plan_destroy(h_out)
+
+
+@pytest.mark.parametrize("seed", range(36))
+def test_random_tensor_lists(q, oracle, seed):
+    """Random lists: row lengths on both sides of every kind boundary of the planner, 1-D and
+    empty tensors, column-strided and row-strided views, group sizes 1 ... 17, both ops, all
+    dtypes; short lists (descriptors in the kernel arguments) and long ones (device table)."""
+    import random
+    rnd = random.Random(1000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    dtype = [torch.float32, torch.bfloat16, torch.float16][seed % 3]
+    ws = rnd.choice([1, 2, 3, 4, 7, 8, 9, 16, 17])
+    op = rnd.choice([ReduceOp.SUM, ReduceOp.AVG])
+    n_tensors = rnd.choice([1, 3, 9, 16, 17, 40])
+    edges = [1, 2, 3, 4, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 260,
+             511, 512, 513, 520, 1023, 1024, 1025, 2047, 2048, 2049, 4095, 4096, 4100, 8191, 8192, 8200]
+
+    def one_tensor():
+        kind = rnd.random()
+        n = rnd.choice(edges) if rnd.random() < 0.8 else rnd.randint(1, 9000)
+        m = rnd.choice([0, 1, 2, 5, 16, 33, 70]) if n > 512 else rnd.choice([0, 1, 7, 64, 300, 1100])
+        if kind < 0.1:
+            return torch.randn(rnd.choice([1, 5, 1000, 4097]), generator=g)           # 1-D
+        if kind < 0.2:
+            return torch.randn(n, max(m, 1), generator=g).t()                           # column-strided
+        if kind < 0.3:
+            return torch.randn(max(m, 1), n + rnd.randint(1, 9), generator=g)[:, :n]    # row stride > n
+        if kind < 0.35:
+            return torch.randn(max(m, 1) * n + 1, generator=g)[1:].view(max(m, 1), n)   # element-aligned base
+        return torch.randn(m, n, generator=g)
+
+    protos = [one_tensor() for _ in range(n_tensors)]
+    peers = []
+    for p in range(ws):
+        ts = []
+        for t in protos:
+            x = torch.randn(t.shape, generator=g) * (10.0 ** rnd.randint(-4, 3))
+            if x.numel() > 8:
+                x.view(-1)[3] = 0.0
+            y = torch.empty_strided(t.shape, t.stride(), dtype=dtype) if t.numel() else torch.empty(t.shape, dtype=dtype)
+            y.copy_(x)
+            ts.append(y)
+        peers.append(ts)
+    ranks = None if ws <= 4 else sorted({0, rnd.randrange(ws), ws - 1})
+    full_check(q, oracle, peers, ws, op, ranks)
