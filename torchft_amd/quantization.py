@@ -150,8 +150,36 @@ def _prepare(inputs: list[torch.Tensor], all_reduce_group_size: int) -> tuple[_P
     return plan, device
 
 
+# Per-call host cost matters for the per-parameter all-reduce (thousands of small
+# calls): the raw current stream and the current device come from torch's C
+# bindings where they exist (0.3 us instead of 4 us for a Stream object and
+# 2 us for a device context that changes nothing).
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream_ptr(device: torch.device) -> ctypes.c_void_p:
+    if _raw_stream is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device: torch.device):
+    """Context in which ``device`` is the current device."""
+    if _raw_device is not None and device.index is not None and _raw_device() == device.index:
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _check_packed(output: torch.Tensor, plan: _Plan) -> None:
@@ -164,7 +192,7 @@ def _check_packed(output: torch.Tensor, plan: _Plan) -> None:
 # call these; torchft_amd.collectives prepares once per collective and calls
 # all three, which saves two walks over the tensor list.
 def _quantize(plan: _Plan, device: torch.device) -> torch.Tensor:
-    with torch.cuda.device(device):
+    with _on_device(device):
         # float32 storage like the reference (:567-571) so that scales are aligned
         output = torch.empty(plan.output_size // SCALE_DTYPE_BYTES, device=device,
                              dtype=SCALE_DTYPE).view(torch.uint8)
@@ -177,7 +205,7 @@ def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
             reduce_op: ReduceOp) -> None:
     _check_packed(output, plan)
     is_avg = 0 if reduce_op == ReduceOp.SUM else 1  # anything but SUM averages (:682)
-    with torch.cuda.device(device):
+    with _on_device(device):
         _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
                                      plan.output_size, int(rank), is_avg,
                                      _stream_ptr(device)), "tftq_reduce")
@@ -185,7 +213,7 @@ def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
 
 def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor) -> None:
     _check_packed(output, plan)
-    with torch.cuda.device(device):
+    with _on_device(device):
         _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
                                          plan.output_size, _stream_ptr(device)),
                "tftq_dequantize")
