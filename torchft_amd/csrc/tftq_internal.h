@@ -10,23 +10,25 @@
 enum : int { ST_Q = 0, ST_R = 1, ST_D = 2 };
 
 // How the rows of one tensor are mapped onto lanes.  "Team" = the lanes that
-// cooperate on one row.  VEC kinds need contiguous 16-byte aligned rows whose
-// length is a whole number of 16-byte vectors; GEN kinds take any strides.
+// cooperate on one row.  VEC kinds (quantize, dequantize) need rows that are
+// contiguous in memory (column stride 1; any row stride, any element-aligned
+// start, any length); GEN kinds take any strides there.  In reduce every row of
+// the packed buffer is contiguous and the GEN kinds only differ in team size.
 enum : uint8_t {
     K_NONE = 0,
+    K_VECS = 13,   // rows of 1-32 whole 16-byte vectors: 1 to 8 lanes per row, several rows per lane
     K_VEC8 = 1,    // 8 lanes per row, 32 rows per workgroup
+    K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
+    K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
     K_VEC64 = 2,   // one wavefront per row, 4 rows per workgroup
     K_VEC256 = 3,  // one workgroup per row (also loops over rows too long for registers)
     K_GEN1 = 4,    // one lane per row, 256 rows per workgroup
     K_GEN8 = 5,    // 8 lanes per row
+    K_GEN16 = 9,   // 16 lanes per row (reduce only)
+    K_GEN32 = 10,  // 32 lanes per row (reduce only)
     K_GEN64 = 6,   // one wavefront per row
     K_GEN256 = 7,  // one workgroup per row (reduce only)
     K_COL1 = 8,    // rows of a single column (1-D tensors): 4 rows per lane, 1024 per workgroup
-    K_GEN16 = 9,   // 16 lanes per row (reduce only)
-    K_GEN32 = 10,  // 32 lanes per row (reduce only)
-    K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
-    K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
-    K_VECS = 13,   // contiguous rows of at most 32 whole vectors: 1 to 8 lanes per row, several rows per lane
 };
 
 static inline int tftq_team_of(uint8_t kind)
@@ -91,7 +93,7 @@ struct Seg {
     int32_t row_bytes;   // 4 + round_up(n, 4)
     int32_t wg_begin[3]; // first workgroup of this segment, per stage
     uint8_t kind[3];     // lane mapping, per stage
-    uint8_t reduce_rows_per_team;  // reduce: consecutive rows one team works through (wide teams)
+    uint8_t reduce_rows_per_team;  // reduce: consecutive rows one team of 64 or 256 lanes works through (1 today)
 };
 static_assert(sizeof(Seg) == 64, "Seg must be 64 bytes");
 
