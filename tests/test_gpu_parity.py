@@ -641,3 +641,23 @@ def test_random_tensor_lists(q, oracle, seed):
         peers.append(ts)
     ranks = None if ws <= 4 else sorted({0, rnd.randrange(ws), ws - 1})
     full_check(q, oracle, peers, ws, op, ranks)
+
+
+def test_plan_cache_eviction(q, oracle, monkeypatch):
+    """Plans are dropped from the cache while their kernels may still be queued; results
+    stay correct and the cache stays within its limits."""
+    monkeypatch.setattr(q, "_PLAN_CACHE_SIZE", 3)
+    monkeypatch.setattr(q, "_PLAN_CACHE_TENSORS", 60)
+    g = torch.Generator().manual_seed(5)
+    ws = 2
+    lists = []
+    for k in range(8):
+        n = 1 if k % 2 else 25  # single tensors and lists long enough for a device table
+        lists.append([torch.randn(9 + k, 40 + 3 * j, generator=g) for j in range(n)])
+    packed = []
+    for _ in range(3):
+        packed = [q.fused_quantize_into_fp8(dev(ts), ws) for ts in lists]  # no synchronisation in between
+    torch.cuda.synchronize()
+    assert len(q._plan_cache) <= 3 and q._plan_cache_tensors <= 60
+    for ts, got in zip(lists, packed):
+        same_bytes(got, oracle.fused_quantize_into_fp8(list(ts), ws), "quantize after eviction")

@@ -38,18 +38,23 @@ SCALE_DTYPE_BYTES: int = 4
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 _TENSOR = torch.Tensor
 _DTYPE_OF = operator.attrgetter("dtype")
-_PLAN_CACHE_SIZE = 64
+# Plans are cached by (device, dtype, group size, addresses, shapes, strides).  The
+# per-parameter all-reduce of a model has one single-tensor plan per parameter, so the
+# cache holds thousands of small plans; long lists are bounded by their total length.
+_PLAN_CACHE_SIZE = 4096
+_PLAN_CACHE_TENSORS = 1 << 18
 
 
 class _Plan:
     """Owns a ``tftq_plan`` and, for long tensor lists, its device table."""
 
-    __slots__ = ("handle", "output_size", "slot_size", "max_rows", "table", "_lib")
+    __slots__ = ("handle", "output_size", "slot_size", "max_rows", "table", "n_tensors", "_lib")
 
-    def __init__(self, lib, handle, table):
+    def __init__(self, lib, handle, table, n_tensors):
         self._lib = lib
         self.handle = handle
         self.table = table
+        self.n_tensors = n_tensors
         self.output_size = lib.tftq_plan_output_size(handle)
         self.slot_size = lib.tftq_plan_slot_size(handle)
         self.max_rows = lib.tftq_plan_max_rows(handle)
@@ -65,6 +70,7 @@ class _Plan:
 
 _cache_lock = threading.Lock()
 _plan_cache: "OrderedDict[tuple, _Plan]" = OrderedDict()
+_plan_cache_tensors = 0
 
 
 def _check(rc: int, what: str) -> None:
@@ -142,11 +148,18 @@ def _prepare(inputs: list[torch.Tensor], all_reduce_group_size: int) -> tuple[_P
         table = torch.frombuffer(host, dtype=torch.uint8).to(device)
         _check(lib.tftq_plan_set_device_table(handle, ctypes.c_void_p(table.data_ptr())),
                "tftq_plan_set_device_table")
-    plan = _Plan(lib, handle, table)
+    plan = _Plan(lib, handle, table, T)
+    global _plan_cache_tensors
     with _cache_lock:
+        old = _plan_cache.pop(key, None)  # another thread may have built the same plan
+        if old is not None:
+            _plan_cache_tensors -= old.n_tensors
         _plan_cache[key] = plan
-        while len(_plan_cache) > _PLAN_CACHE_SIZE:
-            _plan_cache.popitem(last=False)
+        _plan_cache_tensors += T
+        while len(_plan_cache) > 1 and (len(_plan_cache) > _PLAN_CACHE_SIZE
+                                        or _plan_cache_tensors > _PLAN_CACHE_TENSORS):
+            _, gone = _plan_cache.popitem(last=False)
+            _plan_cache_tensors -= gone.n_tensors
     return plan, device
 
 
@@ -182,6 +195,13 @@ def _on_device(device: torch.device):
     return torch.cuda.device(device)
 
 
+def _keep_table(plan: _Plan, device: torch.device) -> None:
+    """A plan can be evicted from the cache while its kernel is still queued: tell the
+    allocator on which stream the device table is in use."""
+    if plan.table is not None:
+        plan.table.record_stream(torch.cuda.current_stream(device))
+
+
 def _check_packed(output: torch.Tensor, plan: _Plan) -> None:
     assert output.shape[0] == plan.output_size, "Output size does not match"
     if output.dtype != torch.uint8 or not output.is_contiguous():
@@ -198,6 +218,7 @@ def _quantize(plan: _Plan, device: torch.device) -> torch.Tensor:
                              dtype=SCALE_DTYPE).view(torch.uint8)
         _check(plan._lib.tftq_quantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
                                        plan.output_size, _stream_ptr(device)), "tftq_quantize")
+        _keep_table(plan, device)
     return output
 
 
@@ -209,6 +230,7 @@ def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
         _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
                                      plan.output_size, int(rank), is_avg,
                                      _stream_ptr(device)), "tftq_reduce")
+        _keep_table(plan, device)
 
 
 def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor) -> None:
@@ -217,6 +239,7 @@ def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor) -> None
         _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
                                          plan.output_size, _stream_ptr(device)),
                "tftq_dequantize")
+        _keep_table(plan, device)
 
 
 def fused_quantize_into_fp8(
