@@ -45,7 +45,7 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
 // Contiguous, 16-byte aligned rows.  Four vectors per lane and step; their loads
 // are issued together without a branch (lanes past the end re-read the last
 // vector and do not store).
-template <typename T, int TEAM, bool NT>
+template <typename T, int TEAM, bool NT, int DV>
 DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
 {
     if (row >= s.m) return;
@@ -56,7 +56,6 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
         return;
     }
     constexpr int EPV = Elem<T>::EPV;
-    constexpr int DV = 8;  // loads in flight per lane (4: 1.3 % slower on 4096-column bf16 rows)
     const int nvec = s.n / EPV;
     GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
     // the few columns after the last whole vector, one element per lane
@@ -101,8 +100,16 @@ template <typename T, int TEAM>
 DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
 {
     // same branch for the whole workgroup
-    if (rows_fill_lines<T>(s)) dequantize_vec_nt<T, TEAM, true>(s, p, row, lane);
-    else dequantize_vec_nt<T, TEAM, false>(s, p, row, lane);
+    // DV = vectors a lane loads per step: 8 in flight where the row has them (4 is 1.3 % slower
+    // on 4096-column bf16 rows), 4 for shorter rows, whose lanes would mostly load duplicates
+    const bool few = s.n / Elem<T>::EPV <= 4 * TEAM;
+    if (rows_fill_lines<T>(s)) {
+        if (few) dequantize_vec_nt<T, TEAM, true, 4>(s, p, row, lane);
+        else dequantize_vec_nt<T, TEAM, true, 8>(s, p, row, lane);
+    } else {
+        if (few) dequantize_vec_nt<T, TEAM, false, 4>(s, p, row, lane);
+        else dequantize_vec_nt<T, TEAM, false, 8>(s, p, row, lane);
+    }
 }
 
 // Rows of one column: one plain divide per row, four rows per lane.
@@ -125,11 +132,11 @@ DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 
 // K_VECS in dequantize: same shape as quantize_small, 8 vectors of codes and their
 // rows' scales in flight per lane.
-template <typename T, int LC, bool NT>
+template <typename T, int C, bool NT>
 DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
 {
     constexpr int EPV = Elem<T>::EPV;
-    constexpr int C = 1 << LC, ROWS = 8 >> LC;
+    constexpr int ROWS = 8 / C;
     const int nvec = s.n / EPV;
     const int row0 = blk * (h.teams * ROWS);
     const float inv = 1.0f / (float)s.slice_rows;
@@ -196,13 +203,15 @@ DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid)
 {
     const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
     if (rows_fill_lines<T>(s)) {
-        if (h.lc == 0) dequantize_small_c<T, 0, true>(s, p, blk, tid, h);
-        else if (h.lc == 1) dequantize_small_c<T, 1, true>(s, p, blk, tid, h);
-        else dequantize_small_c<T, 2, true>(s, p, blk, tid, h);
+        if (h.c == 1) dequantize_small_c<T, 1, true>(s, p, blk, tid, h);
+        else if (h.c == 2) dequantize_small_c<T, 2, true>(s, p, blk, tid, h);
+        else if (h.c == 3) dequantize_small_c<T, 3, true>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 4, true>(s, p, blk, tid, h);
     } else {
-        if (h.lc == 0) dequantize_small_c<T, 0, false>(s, p, blk, tid, h);
-        else if (h.lc == 1) dequantize_small_c<T, 1, false>(s, p, blk, tid, h);
-        else dequantize_small_c<T, 2, false>(s, p, blk, tid, h);
+        if (h.c == 1) dequantize_small_c<T, 1, false>(s, p, blk, tid, h);
+        else if (h.c == 2) dequantize_small_c<T, 2, false>(s, p, blk, tid, h);
+        else if (h.c == 3) dequantize_small_c<T, 3, false>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 4, false>(s, p, blk, tid, h);
     }
 }
 

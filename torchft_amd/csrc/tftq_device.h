@@ -382,15 +382,14 @@ DEV int64_t row_addr(const Seg &s, int64_t slot_size, int row)
 // row0 + r * teams + t: for a given r the teams of a wavefront read
 // consecutive rows, i.e. consecutive memory.
 struct SmallShape {
-    int lt, lc, team, teams, nrow, t, l;
+    int lt, c, team, teams, t, l;
 };
 DEV SmallShape small_shape(int nvec, int tid)
 {
     SmallShape h;
-    tftq_small_shape(nvec, &h.lt, &h.lc);
+    tftq_small_shape(nvec, &h.lt, &h.c);
     h.team = 1 << h.lt;
     h.teams = TFTQ_WG >> h.lt;
-    h.nrow = 8 >> h.lc;
     h.t = tid >> h.lt;
     h.l = tid & (h.team - 1);
     return h;

@@ -54,22 +54,24 @@ constexpr int TFTQ_WG = 256;       // threads per workgroup, all kernels
 #endif
 
 // K_VECS: a row of nvec (1..32) 16-byte vectors is owned by a team of 2^lt lanes
-// (1, 2, 4 or 8), every lane holds 2^lc (1, 2 or 4) vectors of it, and works on
-// 8 >> lc rows at once, so that it has 8 loads in flight whatever the row length.
-TFTQ_HD static inline void tftq_small_shape(int nvec, int *lt, int *lc)
+// (the smallest of 1, 2, 4, 8 that holds it with one vector per lane, else 8),
+// every lane holds c (1 to 4) vectors of it and works on 8 / c rows at once, so
+// that it has 6 to 8 loads in flight whatever the row length.  (Smaller teams
+// with more vectors per lane would leave fewer idle slots for some lengths,
+// 9 vectors as 4 x 3 for example, but measured slower: their loads cover
+// shorter runs of memory.)
+TFTQ_HD static inline void tftq_small_shape(int nvec, int *lt, int *c)
 {
-    int t = 0, c = 0;
+    int t = 0;
     while (t < 3 && (1 << t) < nvec) t++;
-    const int per_lane = (nvec + (1 << t) - 1) >> t;
-    while ((1 << c) < per_lane) c++;
     *lt = t;
-    *lc = c;
+    *c = (nvec + (1 << t) - 1) >> t;
 }
 static inline int tftq_small_rows_per_wg(int nvec)
 {
-    int lt, lc;
-    tftq_small_shape(nvec, &lt, &lc);
-    return (TFTQ_WG >> lt) * (8 >> lc);
+    int lt, c;
+    tftq_small_shape(nvec, &lt, &c);
+    return (TFTQ_WG >> lt) * (8 / c);
 }
 constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
 

@@ -226,11 +226,11 @@ DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 }
 
 // Short contiguous rows of whole 16-byte vectors (K_VECS, shape in tftq_device.h).
-template <typename T, int LC>
+template <typename T, int C>
 DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
 {
     constexpr int EPV = Elem<T>::EPV;
-    constexpr int C = 1 << LC, ROWS = 8 >> LC;  // vectors per lane and row, rows per lane
+    constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane
     const int nvec = s.n / EPV;
     const int row0 = blk * (h.teams * ROWS);
     const int m_pad = s.slice_rows * p.ws;
@@ -273,9 +273,10 @@ template <typename T>
 DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid)
 {
     const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
-    if (h.lc == 0) quantize_small_c<T, 0>(s, p, blk, tid, h);
-    else if (h.lc == 1) quantize_small_c<T, 1>(s, p, blk, tid, h);
-    else quantize_small_c<T, 2>(s, p, blk, tid, h);
+    if (h.c == 1) quantize_small_c<T, 1>(s, p, blk, tid, h);
+    else if (h.c == 2) quantize_small_c<T, 2>(s, p, blk, tid, h);
+    else if (h.c == 3) quantize_small_c<T, 3>(s, p, blk, tid, h);
+    else quantize_small_c<T, 4>(s, p, blk, tid, h);
 }
 
 template <typename T, bool INLINE, bool WIDE>
