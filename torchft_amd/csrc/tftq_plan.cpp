@@ -53,7 +53,7 @@ extern "C" int tftq_layout(int n_tensors, const int64_t *shapes, int ws, int64_t
     return 0;
 }
 
-static uint8_t pick_io_kind(const Seg &s, int esz, int st)
+static uint8_t pick_io_kind(const Seg &s, int esz)
 {
     // Vector kinds: contiguous rows of at least 64 bytes.  Neither the row start nor the
     // row length needs to be a multiple of 16 bytes: gfx950 loads and stores 16-byte
@@ -65,13 +65,13 @@ static uint8_t pick_io_kind(const Seg &s, int esz, int st)
     if (s.ptr != 0 && s.col_stride == 1 && s.n % epv == 0 && s.n / epv >= 1 && s.n / epv <= 32)
         return K_VECS;  // short rows of whole vectors
     if (vec_ok) {
-        // 2 to 4 vectors of 16 bytes per lane (dequantize: up to 8 with 32 lanes), 8 in a
-        // wavefront's row before a whole workgroup takes it.  Measured on MI355X: 1000-column
-        // bf16 rows quantize at 6.6 TB/s with 32 lanes per row, 5.7 with 16 and 6.3 with 64;
-        // 4 KB rows dequantize 1 to 4 % faster with 32 lanes than with 64.
+        // Team sizes measured on MI355X inside quantize -> reduce -> dequantize sequences (a
+        // kernel's time depends on what ran before it, so loops over one kernel mislead):
+        // 528-byte rows are fastest with 16 lanes, 1 to 4 KB rows with 32 (1000-column bf16
+        // rows: 303 us per sequence against 346 us with 16 lanes), longer ones with 64.
         if (in_bytes <= 512) return K_VEC8;
         if (in_bytes <= 1024) return K_VEC16;
-        if (in_bytes <= (st == ST_D ? 4096 : 2048)) return K_VEC32;
+        if (in_bytes <= 4096) return K_VEC32;
         if (in_bytes <= 8192) return K_VEC64;
         return K_VEC256;  // longer than 32 KB: two passes inside the workgroup
     }
@@ -282,8 +282,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         const int64_t m_pad = (int64_t)s.slice_rows * ws;
         if (m_pad > p->max_rows) p->max_rows = m_pad;
 
-        s.kind[ST_Q] = pick_io_kind(s, p->esz, ST_Q);
-        s.kind[ST_D] = pick_io_kind(s, p->esz, ST_D);
+        s.kind[ST_Q] = s.kind[ST_D] = pick_io_kind(s, p->esz);
         s.kind[ST_R] = pick_reduce_kind(s);
         s.reduce_rows_per_team = (uint8_t)pick_reduce_rows(s, ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
