@@ -75,7 +75,11 @@ def test_bucket_packing_follows_the_reference(sizes, per_bucket):
 
 
 def test_reference_bucket_walkthroughs():
-    # worked by hand from local_sgd.py:519-553
+    # worked by hand from local_sgd.py:519-553; the module's planner and this file's restatement
+    for sizes, cap in (([6, 6, 6, 6], 8), ([2, 9, 2], 8), ([3, 5, 4], 8), ([1] * 17, 4), ([10, 10, 10], 1000)):
+        assert A.plan_buckets(sizes, cap) == reference_buckets(sizes, cap)
+    assert A.plan_buckets([6, 6, 6, 6], 8) == [(8, [0]), (8, [1]), (8, [2])]
+    assert A.plan_buckets([2, 9, 2], 8) == [(8, [0]), (5, [])]
     # four tensors of 6 elements, buckets of 8: one tensor per bucket, the offset reaches
     # the total (24) after three buckets, the fourth tensor is never packed
     assert reference_buckets([6, 6, 6, 6], 8) == [(8, [0]), (8, [1]), (8, [2])]

@@ -147,6 +147,29 @@ def allreduce_per_param(grads: dict, allreduce_fn: Callable[[torch.Tensor], Any]
     return [allreduce_fn(g) for g in grads.values()]
 
 
+def plan_buckets(sizes: list, capacity: int) -> list:
+    """Which tensors share a flat buffer: ``[(buffer length, [tensor indices]), ...]``.
+
+    The reference's walk (local_sgd.py:519-553): a buffer has ``capacity`` elements, or
+    what is left of the total if that is less; tensors are taken in order while they fit;
+    the walk ends when the buffer lengths add up to the total element count.  Because the
+    lengths, not the packed elements, are added up, a tensor that does not fit the rest of
+    a buffer can leave the last tensors in no buffer at all.
+    """
+    total = sum(sizes)
+    plan, covered, nxt = [], 0, 0
+    while covered < total:
+        length = min(capacity, total - covered)
+        members, used = [], 0
+        while nxt < len(sizes) and used + sizes[nxt] <= length:
+            members.append(nxt)
+            used += sizes[nxt]
+            nxt += 1
+        plan.append((length, members))
+        covered += length
+    return plan
+
+
 def bucketize_and_allreduce(
     tensors: list,
     bucket_size_bytes: int,
@@ -158,53 +181,39 @@ def bucketize_and_allreduce(
     (local_sgd.py:499-556) and return the works; each tensor holds its reduced
     values once its bucket's work has been waited on.
 
-    The packing is the reference's, including its corner: the running offset
-    advances by the bucket capacity, not by what was packed (:553), so when a
-    tensor does not fit into the space left in a bucket the loop can end before
-    the last tensors have been packed; those keep their local values.  A
-    bucket capacity that is a multiple of every tensor's size, or larger than
-    the whole list, avoids it.
+    The packing is the reference's (:func:`plan_buckets`), including its corner: tensors
+    that end up in no buffer keep their local values.  A bucket capacity that is a multiple
+    of every tensor's size, or larger than the whole list, avoids it.
 
     ``allreduce_fn(flat)`` is, for example,
     ``lambda t: allreduce(t, pg, n, should_quantize=True)``.
     """
-    works: list = []
     if not tensors:
-        return works
+        return []
+    first = tensors[0]
+    capacity = bucket_size_bytes // first.element_size()
+    assert capacity > 0, "bucket_size_bytes is smaller than one element"
 
-    total_size = sum(t.numel() for t in tensors)
-    dtype, device = tensors[0].dtype, tensors[0].device
-    per_bucket = bucket_size_bytes // tensors[0].element_size()
-    assert per_bucket > 0, "bucket_size_bytes is smaller than one element"
-
-    offset = 0
-    flat_index = 0
-    while offset < total_size:
-        chunk_size = min(per_bucket, total_size - offset)
-        alloc = chunk_size
+    works = []
+    for length, members in plan_buckets([t.numel() for t in tensors], capacity):
+        padded = length
         if row_width:
-            alloc = -(-chunk_size // row_width) * row_width  # whole rows; the tail stays zero
-        flat_buffer = torch.zeros(alloc, dtype=dtype, device=device)
+            padded = -(-length // row_width) * row_width  # whole rows; the tail stays zero
+        flat = torch.zeros(padded, dtype=first.dtype, device=first.device)  # zero-filled (:527-529)
+        spans, at = [], 0
+        for i in members:
+            n = tensors[i].numel()
+            flat[at:at + n].copy_(tensors[i].view(-1))
+            spans.append((tensors[i], at, n))
+            at += n
 
-        pack_offset = 0
-        bucket_tensors: list = []
-        for t in tensors[flat_index:]:
-            numel = t.numel()
-            if pack_offset + numel > chunk_size:
-                break
-            flat_buffer[pack_offset:pack_offset + numel].copy_(t.view(-1))
-            bucket_tensors.append((t, pack_offset, numel))
-            pack_offset += numel
-            flat_index += 1
+        work = allreduce_fn(flat.view(-1, row_width) if row_width else flat)
 
-        work = allreduce_fn(flat_buffer.view(-1, row_width) if row_width else flat_buffer)
-
-        def unpack(fut, bucket_tensors=bucket_tensors, flat_buffer=flat_buffer):
-            for t, pack_offset, numel in bucket_tensors:
-                t.copy_(flat_buffer[pack_offset:pack_offset + numel].view_as(t))
+        def unpack(fut, spans=spans, flat=flat):
+            for t, at, n in spans:
+                t.copy_(flat[at:at + n].view_as(t))
             return []
 
         work.get_future().then(unpack)
         works.append(work)
-        offset += chunk_size
     return works
