@@ -359,6 +359,8 @@ def test_extreme_scales_and_denormals(q, oracle):
 
 
 def test_empty_and_ragged(q, oracle):
+    only_empty = [[torch.zeros(0, 64)], [torch.zeros(0, 64)]]  # empty packed buffer, nothing to launch
+    full_check(q, oracle, only_empty, 2, ReduceOp.AVG)
     peers = [[torch.zeros(0, 5), torch.ones(3, 0), torch.arange(7.0), torch.ones(1, 1)] for _ in range(2)]
     full_check(q, oracle, peers, 2, ReduceOp.SUM)
     full_check(q, oracle, peers * 2, 4, ReduceOp.AVG)
@@ -598,7 +600,7 @@ def test_entry_points_under_graph_capture(q, n_tensors):
     L.tftq_plan_destroy(h_out)
 
 
-@pytest.mark.parametrize("seed", range(36))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TFTQ_RANDOM_LISTS", "36"))))
 def test_random_tensor_lists(q, oracle, seed):
     """Random lists: row lengths on both sides of every kind boundary of the planner, 1-D and
     empty tensors, column-strided and row-strided views, group sizes 1 ... 17, both ops, all

@@ -428,8 +428,10 @@ static inline void work_mapping(const tftq_plan *plan, int stage, KParams *kp)
 static inline int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t packed_bytes,
                        KParams *kp, InlineTable *inl, bool *use_inline)
 {
-    if (!plan || !packed) return TFTQ_E_ARG;
+    if (!plan) return TFTQ_E_ARG;
     if (packed_bytes != plan->output_size) return TFTQ_E_SIZE;
+    // a list of empty tensors has an empty packed buffer, whose address may be null
+    if (!packed && plan->output_size != 0) return TFTQ_E_ARG;
     if (((uintptr_t)packed & 3) != 0) return TFTQ_E_ARG;
     *use_inline = plan->nseg <= TFTQ_N_INLINE;
     if (!*use_inline && !plan->device_table) return TFTQ_E_NOTABLE;
