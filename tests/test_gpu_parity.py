@@ -663,3 +663,31 @@ def test_plan_cache_eviction(q, oracle, monkeypatch):
     assert len(q._plan_cache) <= 3 and q._plan_cache_tensors <= 60
     for ts, got in zip(lists, packed):
         same_bytes(got, oracle.fused_quantize_into_fp8(list(ts), ws), "quantize after eviction")
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TFTQ_RANDOM_EXTREMES", "12"))))
+def test_random_extremes(q, oracle, seed):
+    """Random lists at the far ends: group sizes up to 70, rows of up to 40 000 columns,
+    magnitudes from 1e-38 to 1e38 (scales outside the range of the fast division), zero rows."""
+    import random
+    rnd = random.Random(5000 + seed)
+    g = torch.Generator().manual_seed(5000 + seed)
+    dtype = [torch.float32, torch.bfloat16, torch.float16][seed % 3]
+    ws = rnd.choice([2, 5, 8, 31, 33, 64, 65, 70])
+    op = rnd.choice([ReduceOp.SUM, ReduceOp.AVG])
+    shapes = []
+    for _ in range(rnd.choice([1, 4, 17])):
+        n = rnd.choice([1, 5, 40, 130, 500, 1028, 4100, 9000, 16385, 20000, 32768, 32769, 40000])
+        shapes.append((rnd.choice([1, 2, ws, ws + 1, 3 * ws - 1]) if n > 2000 else rnd.choice([1, 9, 150]), n))
+    top = 4 if dtype == torch.float16 else 37
+    peers = []
+    for p in range(ws):
+        ts = []
+        for (m, n) in shapes:
+            mags = 10.0 ** torch.randint(-top, top, (m, 1), generator=g).float()
+            x = torch.randn(m, n, generator=g).clamp(-3, 3) / 3 * mags
+            if m > 1:
+                x[rnd.randrange(m)] = 0.0
+            ts.append(x.to(dtype))
+        peers.append(ts)
+    full_check(q, oracle, peers, ws, op, ranks=sorted({0, rnd.randrange(ws), ws - 1}))
