@@ -216,7 +216,8 @@ DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
         if (row < m_pad) {
             u32x2 o = {0u, 0u};  // padding rows stay zero
             if (row < s.m) {
-                const float sc = calc_scale(__builtin_fabsf(x[k]));
+                // maximum with 0 as for longer rows: a NaN element is ignored (:131-143)
+                const float sc = calc_scale(fmaxf(0.0f, __builtin_fabsf(x[k])));
                 o.x = as_u(sc);
                 o.y = pack_fp8x4(x[k] * sc, 0.0f, 0.0f, 0.0f) & 0xFFu;
             }

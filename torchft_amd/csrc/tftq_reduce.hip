@@ -478,7 +478,7 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         if (j0 + k * TFTQ_WG + tid < s.slice_rows) {
-            const float s2 = calc_scale(__builtin_fabsf(acc[k]) / p.div);
+            const float s2 = calc_scale(fmaxf(0.0f, __builtin_fabsf(acc[k])) / p.div);  // NaN ignored (:331-338)
             u32x2 o;
             o.x = as_u(s2);
             o.y = pack_fp8x4(scale_div<GDIV>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
