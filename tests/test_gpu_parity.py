@@ -526,6 +526,10 @@ def test_wrapper_errors_on_gpu(q):
         q.fused_dequantize_from_fp8(x, buf[:-4], 2)
     with pytest.raises(RuntimeError):
         q.fused_reduce_fp8(x, buf, 2, 2)
+    with pytest.raises(RuntimeError, match="packed buffer is on cpu"):
+        q.fused_reduce_fp8(x, buf.cpu(), 2, 0)
+    with pytest.raises(RuntimeError, match="packed buffer is on cpu"):
+        q.fused_dequantize_from_fp8(x, buf.cpu(), 2)
 
 
 @pytest.mark.parametrize("n_tensors", [3, 20])

@@ -202,10 +202,13 @@ def _keep_table(plan: _Plan, device: torch.device) -> None:
         plan.table.record_stream(torch.cuda.current_stream(device))
 
 
-def _check_packed(output: torch.Tensor, plan: _Plan) -> None:
+def _check_packed(output: torch.Tensor, plan: _Plan, device: torch.device) -> None:
     assert output.shape[0] == plan.output_size, "Output size does not match"
     if output.dtype != torch.uint8 or not output.is_contiguous():
         raise RuntimeError("the packed buffer must be a contiguous uint8 tensor")
+    if output.device != device:
+        # its address would be handed to a kernel on `device`
+        raise RuntimeError(f"the packed buffer is on {output.device}, the tensors are on {device}")
 
 
 # The three stages on a prepared plan.  The public functions below prepare and
@@ -224,7 +227,7 @@ def _quantize(plan: _Plan, device: torch.device) -> torch.Tensor:
 
 def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
             reduce_op: ReduceOp) -> None:
-    _check_packed(output, plan)
+    _check_packed(output, plan, device)
     is_avg = 0 if reduce_op == ReduceOp.SUM else 1  # anything but SUM averages (:682)
     with _on_device(device):
         _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
@@ -234,7 +237,7 @@ def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
 
 
 def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor) -> None:
-    _check_packed(output, plan)
+    _check_packed(output, plan, device)
     with _on_device(device):
         _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
                                          plan.output_size, _stream_ptr(device)),
