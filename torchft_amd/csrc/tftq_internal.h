@@ -95,7 +95,7 @@ struct Seg {
     int32_t row_bytes;   // 4 + round_up(n, 4)
     int32_t wg_begin[3]; // first workgroup of this segment, per stage
     uint8_t kind[3];     // lane mapping, per stage
-    uint8_t reduce_rows_per_team;  // reduce: consecutive rows one team of 64 or 256 lanes works through (1 today)
+    uint8_t reserved;
 };
 static_assert(sizeof(Seg) == 64, "Seg must be 64 bytes");
 

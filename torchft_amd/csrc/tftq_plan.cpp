@@ -93,19 +93,12 @@ static uint8_t pick_reduce_kind(const Seg &s)
     return K_GEN256;
 }
 
-// Reduce: rows one team works through, prefetching the next row while it
-// finishes the current one.  The kernels support it; one row per team measured
-// fastest on MI355X for every row length (1024-column rows, ws 8: 44 us with
-// one row, 49 / 53 / 67 us with 2 / 4 / 8), because independent workgroups keep
-// more loads in flight than one team's pipeline does.
-static int pick_reduce_rows(const Seg &, int) { return 1; }
-
 static int rows_per_wg_of(const Seg &s, int st, int esz)
 {
     if (s.kind[st] == K_COL1) return 4 * TFTQ_WG;
     if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
     const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
-    return st == ST_R ? teams * s.reduce_rows_per_team : teams;
+    return teams;  // one row per team in every stage
 }
 
 // Bytes one workgroup of segment s moves in a stage.
@@ -284,7 +277,6 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
 
         s.kind[ST_Q] = s.kind[ST_D] = pick_io_kind(s, p->esz);
         s.kind[ST_R] = pick_reduce_kind(s);
-        s.reduce_rows_per_team = (uint8_t)pick_reduce_rows(s, ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
             const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st, p->esz));

@@ -68,12 +68,30 @@ DEV float scale_div(float a, float s2, const KParams &p)
     return GDIV ? y / p.div : y * p.inv_div;
 }
 
+// row maximum / div (:340); for a power-of-two div the multiplication by the
+// exact inverse is the same correctly rounded value, subnormal results included
+template <bool GDIV>
+DEV float amax_div(float amax, const KParams &p)
+{
+    return GDIV ? amax / p.div : amax * p.inv_div;
+}
+
 template <bool GDIV>
 DEV u32x4 requant16(const float (&a)[16], float s2, const KParams &p)
 {
     float y[16];
+    // Power-of-two div: s2 * inv_div is exact unless it is subnormal, and then
+    // a * (s2 * inv_div) rounds the same exact product as (a * s2) * inv_div does in two
+    // steps; the two can only differ below 2^-126, where every code is zero anyway.
+    const float sf = s2 * p.inv_div;
+    const bool fold = !GDIV && (sf == 0.0f || __builtin_fabsf(sf) >= 1.17549435e-38f);
+    if (__builtin_amdgcn_ballot_w64(!fold) == 0) {  // one code path per wavefront
 #pragma unroll
-    for (int e = 0; e < 16; e++) y[e] = scale_div<GDIV>(a[e], s2, p);
+        for (int e = 0; e < 16; e++) y[e] = a[e] * sf;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; e++) y[e] = scale_div<GDIV>(a[e], s2, p);
+    }
     u32x4 o;
     o.x = pack_fp8x4(y[0], y[1], y[2], y[3]);
     o.y = pack_fp8x4(y[4], y[5], y[6], y[7]);
@@ -126,7 +144,7 @@ DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float 
         }
         if (pass == 0) {
             amax = team_max<TEAM>(amax, lds);
-            s2 = calc_scale(amax / p.div);
+            s2 = calc_scale(amax_div<GDIV>(amax, p));
         }
     }
     // the own slot's old scale is an input of every lane: write the new one last (:375)
@@ -201,7 +219,7 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
         }
         if (pass == 0) {
             amax = team_max<256>(amax, lds);  // every wavefront has read the old scales by now
-            s2 = calc_scale(amax / p.div);
+            s2 = calc_scale(amax_div<GDIV>(amax, p));
         }
     }
     if (tid == 0) orow[0] = as_u(s2);  // :375
@@ -296,7 +314,7 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 #pragma unroll
         for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
     amax = team_max<TEAM>(amax, lds);
-    const float s2 = calc_scale(amax / p.div);  // :340
+    const float s2 = calc_scale(amax_div<GDIV>(amax, p));  // :340
 
     GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
 #pragma unroll
@@ -307,30 +325,29 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
     if (lane == 0) orow[0] = as_u(s2);  // :375
 }
 
-// Several rows per team, software-pipelined: the codes of the next batch of
-// peers (of this row or of the next row) are in flight while the current batch
-// is accumulated, so a wavefront always has loads outstanding.  A batch is
-// R_VPB 16-byte vectors per lane: R_VPB / UNITS peers of one row.  Loads carry
-// no branch: a lane past the end of the row re-reads the row's last vector, a
+// One row per team, software-pipelined over the peers: the codes of the next
+// batch of peers are in flight while the current batch is accumulated.  A
+// batch is R_VPB 16-byte vectors per lane: R_VPB / UNITS peers.  Loads carry no
+// branch: a lane past the end of the row re-reads the row's last vector, a
 // batch past the last peer re-reads the last peer, and both are ignored later.
 // Needs ws <= min(TEAM, 64) (lane l of a team, or of each of its wavefronts,
-// holds the scale of peer l) and rows of at least one 16-byte vector.  Teams
-// smaller than a wavefront take one row each; a team whose row is past the end
-// (`valid` false) works on the last row and stores nothing, so that the
-// wavefront stays converged for the cross-lane operations.
+// holds the scale of peer l) and rows of at least one 16-byte vector.  A team
+// whose row is past the end (`valid` false) is given the last row and stores
+// nothing, so that the wavefront stays converged for the cross-lane operations.
+// (Several rows per team with prefetch of the next row were slower for every
+// row length: independent workgroups keep more loads in flight.)
 constexpr int R_VPB = 4;
 
 template <int TEAM, int UNITS, bool PIPE, bool GDIV>
-DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane, float *lds, bool valid = true)
+DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds, bool valid = true)
 {
     constexpr int PB = R_VPB / UNITS >= 1 ? R_VPB / UNITS : 1;  // peers per batch
-    if (TEAM >= 64 && nrows <= 0) return;
     const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
     const int ws = p.ws;
-    const int nb = (ws + PB - 1) / PB;  // batches per row
-    const int total = nrows * nb;
+    const int nb = (ws + PB - 1) / PB;  // batches
     const int wlane = TEAM >= 64 ? (int)(threadIdx.x & 63u) : lane;
     const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
 
     // Vector u of this lane starts at dword doff[u].  The last vector of a row whose
     // length is not a multiple of 4 dwords is moved back so that it ends with the row:
@@ -344,26 +361,20 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
         padmask[u] = (doff[u] == ndw - 4 && (s.n & 3)) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
     }
 
+    // lane l: scale of peer min(l, ws - 1), first in the queue of loads
+    const float raw_scale = as_f(peer_row(p, speer, off)[0]);
+
     struct Batch {
         u32x4 w[PB][UNITS];
-        float scale;  // lane l: guarded scale of peer min(l, ws-1) of the batch's row
     };
     Batch A, B;
-
-    int lrow = 0, lbatch = 0;  // next batch to load
-    auto issue = [&](Batch &dst) {
-        const int64_t off = s.slot_off + (int64_t)(j0 + lrow) * s.row_bytes;
-        dst.scale = as_f(peer_row(p, speer, off)[0]);
+    auto issue = [&](Batch &dst, int batch) {
 #pragma unroll
         for (int b = 0; b < PB; b++) {
-            GLOBAL const u32 *pv = peer_row(p, min(lbatch * PB + b, ws - 1), off) + 1;
+            GLOBAL const u32 *pv = peer_row(p, min(batch * PB + b, ws - 1), off) + 1;
 #pragma unroll
             for (int u = 0; u < UNITS; u++)
                 dst.w[b][u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + doff[u]));
-        }
-        if (++lbatch == nb) {
-            lbatch = 0;
-            ++lrow;
         }
     };
 
@@ -372,13 +383,12 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
     for (int u = 0; u < UNITS; u++)
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
-    int crow = 0, cbatch = 0;  // batch being consumed
     float cr = 1.0f, cl = 0.0f;
     bool row_fast = true;
 
-    auto consume = [&](const Batch &src) {
-        if (cbatch == 0) {
-            const float sc = src.scale == 0.0f ? 1.0f : src.scale;  // padding rows (:419)
+    auto consume = [&](const Batch &src, int batch) {
+        if (batch == 0) {
+            const float sc = raw_scale == 0.0f ? 1.0f : raw_scale;  // padding rows (:419)
             const DivCoef c = make_div(sc);
             cr = c.r;
             cl = c.r_lo;
@@ -387,7 +397,7 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
         if (row_fast) {
 #pragma unroll
             for (int b = 0; b < PB; b++) {
-                const int k = cbatch * PB + b;
+                const int k = batch * PB + b;
                 if (k < ws) {
                     const float pr = team_bcast<TEAM>(cr, k), pl = team_bcast<TEAM>(cl, k);
 #pragma unroll
@@ -399,57 +409,48 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j0, int nrows, int lane
                 }
             }
         }
-        if (++cbatch == nb) {
-            const int j = j0 + crow;
-            if (row_fast) {
-                float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
-#pragma unroll
-                for (int u = 0; u < UNITS; u++)
-#pragma unroll
-                    for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
-                amax = team_max<TEAM>(amax, lds);
-                const float s2 = calc_scale(amax / p.div);  // :340
-                const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
-                GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
-#pragma unroll
-                for (int u = 0; u < UNITS; u++) {
-                    const u32x4 o = requant16<GDIV>(acc[u], s2, p);
-                    if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
-                }
-                if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
-            } else if (valid) {
-                reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
-            }
-#pragma unroll
-            for (int u = 0; u < UNITS; u++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
-            cbatch = 0;
-            ++crow;
-        }
     };
 
     if (!PIPE) {  // long rows: one batch in flight keeps the register count down
-        for (int i = 0; i < total; i++) {
-            issue(A);
-            consume(A);
+        for (int i = 0; i < nb; i++) {
+            issue(A, i);
+            consume(A, i);
         }
-        return;
-    }
-    issue(A);
-    int i = 0;
-    for (; i + 2 < total; i += 2) {
-        issue(B);
-        consume(A);
-        issue(A);
-        consume(B);
-    }
-    if (i + 1 < total) {
-        issue(B);
-        consume(A);
-        consume(B);
     } else {
-        consume(A);
+        issue(A, 0);
+        int i = 0;
+        for (; i + 2 < nb; i += 2) {
+            issue(B, i + 1);
+            consume(A, i);
+            issue(A, i + 2);
+            consume(B, i + 1);
+        }
+        if (i + 1 < nb) {
+            issue(B, i + 1);
+            consume(A, i);
+            consume(B, i + 1);
+        } else {
+            consume(A, i);
+        }
+    }
+
+    if (row_fast) {
+        float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
+#pragma unroll
+        for (int u = 0; u < UNITS; u++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+        amax = team_max<TEAM>(amax, lds);
+        const float s2 = calc_scale(amax_div<GDIV>(amax, p));  // :340
+        GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const u32x4 o = requant16<GDIV>(acc[u], s2, p);
+            if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
+        }
+        if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+    } else if (valid) {
+        reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
     }
 }
 
@@ -478,7 +479,7 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         if (j0 + k * TFTQ_WG + tid < s.slice_rows) {
-            const float s2 = calc_scale(fmaxf(0.0f, __builtin_fabsf(acc[k])) / p.div);  // NaN ignored (:331-338)
+            const float s2 = calc_scale(amax_div<GDIV>(fmaxf(0.0f, __builtin_fabsf(acc[k])), p));  // NaN ignored (:331-338)
             u32x2 o;
             o.x = as_u(s2);
             o.y = pack_fp8x4(scale_div<GDIV>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
@@ -497,44 +498,36 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
     const int blk = vb - s.wg_begin[ST_R];
     const int tid = threadIdx.x;
     const int ndw = (s.row_bytes >> 2) - 1;
-    const int rpt = s.reduce_rows_per_team;
     switch (s.kind[ST_R]) {
-    case K_GEN256: {
-        const int j0 = blk * rpt;
-        const int nrows = min(rpt, s.slice_rows - j0);
+    case K_GEN256: {  // one workgroup per row
+        const int j = blk;
         if (WIDE && ndw > TFTQ_R_DWORDS && ndw <= TFTQ_R_DWORDS_WIDE && p.ws <= 64) {
-            reduce_rows<256, 8, false, GDIV>(s, p, j0, nrows, tid, lds);
+            reduce_rows<256, 8, false, GDIV>(s, p, j, tid, lds);
         } else if (ndw > TFTQ_R_DWORDS) {
-            for (int r = 0; r < nrows; r++) {
-                if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j0 + r, tid, lds);
-                else reduce_row_long<GDIV>(s, p, j0 + r, tid, lds);
-            }
+            if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
+            else reduce_row_long<GDIV>(s, p, j, tid, lds);
         } else if (p.ws > 64) {
-            for (int r = 0; r < nrows; r++) {
-                if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j0 + r, tid, lds);
-                else reduce_row<256, 4, GDIV>(s, p, j0 + r, tid, lds);
-            }
+            if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j, tid, lds);
+            else reduce_row<256, 4, GDIV>(s, p, j, tid, lds);
         } else if (ndw <= 1024) {
-            reduce_rows<256, 1, true, GDIV>(s, p, j0, nrows, tid, lds);
+            reduce_rows<256, 1, true, GDIV>(s, p, j, tid, lds);
         } else if (ndw <= 2048) {
-            reduce_rows<256, 2, true, GDIV>(s, p, j0, nrows, tid, lds);
+            reduce_rows<256, 2, true, GDIV>(s, p, j, tid, lds);
         } else {
-            reduce_rows<256, 4, false, GDIV>(s, p, j0, nrows, tid, lds);
+            reduce_rows<256, 4, false, GDIV>(s, p, j, tid, lds);
         }
         break;
     }
-    case K_GEN64: {
-        const int j0 = (blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6)) * rpt;
-        const int nrows = min(rpt, s.slice_rows - j0);
+    case K_GEN64: {  // one wavefront per row
+        const int j = blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);
+        if (j >= s.slice_rows) break;  // the whole wavefront leaves
         if (p.ws > 64) {
-            for (int r = 0; r < nrows; r++) {
-                if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j0 + r, tid & 63, lds);
-                else reduce_row<64, 2, GDIV>(s, p, j0 + r, tid & 63, lds);
-            }
+            if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j, tid & 63, lds);
+            else reduce_row<64, 2, GDIV>(s, p, j, tid & 63, lds);
         } else if (ndw <= 256) {
-            reduce_rows<64, 1, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
+            reduce_rows<64, 1, true, GDIV>(s, p, j, tid & 63, lds);
         } else {
-            reduce_rows<64, 2, true, GDIV>(s, p, j0, nrows, tid & 63, lds);
+            reduce_rows<64, 2, true, GDIV>(s, p, j, tid & 63, lds);
         }
         break;
     }
@@ -546,7 +539,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
             constexpr int TEAM = decltype(team_c)::value;
             const int j = blk * (TFTQ_WG / TEAM) + tid / TEAM;
             if (p.ws <= TEAM) {
-                reduce_rows<TEAM, 1, true, GDIV>(s, p, min(j, s.slice_rows - 1), 1, tid % TEAM, lds, j < s.slice_rows);
+                reduce_rows<TEAM, 1, true, GDIV>(s, p, min(j, s.slice_rows - 1), tid % TEAM, lds, j < s.slice_rows);
             } else {
                 reduce_row<TEAM, 1, GDIV>(s, p, j, tid % TEAM, lds);
             }
