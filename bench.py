@@ -144,7 +144,7 @@ def main() -> int:
         "2": (lambda seed: workloads.cfg2(seed, device=dev), 8, ReduceOp.AVG,
               "config 2: one bf16 tensor [4096, 4096], N(0, 0.02), ws=8, AVG"),
         "3": (lambda seed: workloads.cfg3(seed, device=dev), 8, ReduceOp.AVG,
-              "BASELINE config 3: Llama-3-8B decoder-layer gradient bucket, "
+              "benchmark configuration 3: Llama-3-8B decoder-layer gradient bucket, "
               "9 bf16 tensors, 218112000 elements, ws=8, reduce AVG"),
         "4": (lambda seed: workloads.cfg4(seed, device=dev), 4, ReduceOp.AVG,
               "config 4: DiLoCo pseudo-gradient of a 1.1B model, 201 fp32 tensors, "
