@@ -746,3 +746,56 @@ def test_nan_and_inf_rows(q, oracle, dtype):
             assert torch.equal(torch.nan_to_num(a.float(), nan=0.0), torch.nan_to_num(b.float(), nan=0.0))
             same = ~torch.isnan(a)
             assert torch.equal(torch.signbit(a[same]), torch.signbit(b[same]))
+
+
+def test_concurrent_threads_and_streams(q, oracle):
+    """Eight threads, each on its own stream, hammer the three entry points on shared and on
+    private tensor lists at the same time (one plan cache, one library): every result must be
+    the checker's."""
+    import threading
+    ws, rank = 4, 1
+    g = torch.Generator().manual_seed(11)
+    shared_cpu = [torch.randn(33, 4096, generator=g).to(torch.bfloat16), torch.randn(500, 72, generator=g).to(torch.bfloat16)]
+    shared = dev(shared_cpu)
+    want_q = oracle.fused_quantize_into_fp8(list(shared_cpu), ws)
+    want_r = want_q.clone()
+    oracle.fused_reduce_fp8(list(shared_cpu), want_r, ws, rank, ReduceOp.AVG)
+    errors = []
+
+    def worker(t):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            gg = torch.Generator().manual_seed(100 + t)
+            mine_cpu = [torch.randn(17 + t, 1000 + 8 * t, generator=gg), torch.randn(64 * (t + 1), generator=gg)]
+            mine = dev(mine_cpu)
+            want_mine = oracle.fused_quantize_into_fp8(list(mine_cpu), ws)
+            with torch.cuda.stream(stream):
+                for it in range(40):
+                    a = q.fused_quantize_into_fp8(shared, ws)
+                    b = q.fused_quantize_into_fp8(mine, ws)
+                    r = a.clone()
+                    q.fused_reduce_fp8(shared, r, ws, rank, ReduceOp.AVG)
+                    out = [torch.empty_like(x) for x in mine]
+                    q.fused_dequantize_from_fp8(out, b, ws)
+                    if it % 13 == 0:
+                        stream.synchronize()
+                        assert torch.equal(a.cpu(), want_q) and torch.equal(b.cpu(), want_mine)
+                        assert torch.equal(r.cpu(), want_r)
+                stream.synchronize()
+                assert torch.equal(a.cpu(), want_q) and torch.equal(b.cpu(), want_mine) and torch.equal(r.cpu(), want_r)
+                ref = [torch.empty_like(x) for x in mine_cpu]
+                oracle.fused_dequantize_from_fp8(ref, want_mine, ws)
+                for x, y in zip(out, ref):
+                    same_bytes(x, y, f"thread {t}")
+        except BaseException as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=120)
+        assert not th.is_alive()
+    if errors:
+        raise errors[0]
