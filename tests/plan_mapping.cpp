@@ -114,7 +114,7 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
             else if (s.kind[st] == K_VECS) per_wg = tftq_small_rows_per_wg(s.n / (dtype == TFTQ_F32 ? 4 : 8));
             else {
                 const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
-                per_wg = teams;
+                per_wg = st == ST_R ? teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws) : teams;
             }
             const int64_t blocks = (rows + per_wg - 1) / per_wg;
             seen[(size_t)i].assign((size_t)blocks, 0);

@@ -260,6 +260,31 @@ def test_group_sizes(q, oracle, ws, op):
     full_check(q, oracle, peers, ws, op, ranks)
 
 
+@pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (2, ReduceOp.AVG), (2, ReduceOp.SUM), (3, ReduceOp.AVG),
+                                   (4, ReduceOp.AVG), (4, ReduceOp.SUM)])
+def test_small_groups_several_rows_at_once(q, oracle, ws, op):
+    """Groups of up to four peers: a team of 64 or 256 lanes reduces two or four rows at
+    once.  Row lengths on both sides of every team/vector-count boundary, rows per slot
+    that are not multiples of two or four (1, 2, 3, 5, 7, 9), a zero row and a row whose
+    scale needs the plain divide in the middle of a set."""
+    g = torch.Generator().manual_seed(300 + ws)
+    cols = [516, 600, 1024, 1028, 1500, 2048, 2052, 3000, 4096, 4100, 6000, 8192, 8196, 9000]
+    slot_rows = [1, 2, 3, 5, 7, 9]
+    shapes = [(slot_rows[i % 6] * ws - (i % 2 if ws > 1 else 0), c) for i, c in enumerate(cols)]
+    peers = []
+    for p in range(ws):
+        ts = []
+        for r, c in shapes:
+            x = torch.randn(r, c, generator=g) * (1 + p)
+            if r > 1:
+                x[1] *= 1e-30
+            if r > 2:
+                x[2] = 0.0
+            ts.append(x.to(torch.bfloat16))
+        peers.append(ts)
+    full_check(q, oracle, peers, ws, op)
+
+
 @pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (16, ReduceOp.AVG), (24, ReduceOp.SUM),
                                    (40, ReduceOp.AVG)])
 def test_short_rows_all_team_sizes(q, oracle, ws, op):

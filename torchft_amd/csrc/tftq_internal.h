@@ -31,7 +31,14 @@ enum : uint8_t {
     K_COL1 = 8,    // rows of a single column (1-D tensors): 4 rows per lane, 1024 per workgroup
 };
 
-static inline int tftq_team_of(uint8_t kind)
+// Helpers shared by the planner (host compiler) and the kernels (hipcc).
+#ifdef __HIPCC__
+#define TFTQ_HD __host__ __device__
+#else
+#define TFTQ_HD
+#endif
+
+TFTQ_HD static inline int tftq_team_of(uint8_t kind)
 {
     switch (kind) {
     case K_VEC8: case K_GEN8: return 8;
@@ -46,12 +53,18 @@ static inline int tftq_team_of(uint8_t kind)
 
 constexpr int TFTQ_WG = 256;       // threads per workgroup, all kernels
 
-// Helpers shared by the planner (host compiler) and the kernels (hipcc).
-#ifdef __HIPCC__
-#define TFTQ_HD __host__ __device__
-#else
-#define TFTQ_HD
-#endif
+// Reduce, teams of 64 or 256 lanes: a lane has 8 loads of 16 bytes in flight
+// when the group has 8 peers.  With fewer peers a team works on 2 or 4
+// consecutive rows at once so that it still has (ws = 2: 2 -> 8 loads per lane).
+TFTQ_HD static inline int tftq_reduce_rows_at_once(uint8_t kind, int ndw, int ws)
+{
+    if (kind != K_GEN256 && kind != K_GEN64) return 1;
+    const int unit_dw = tftq_team_of(kind) * 4;  // dwords that one vector per lane covers
+    const int units = (ndw + unit_dw - 1) / unit_dw;  // vectors per lane and peer
+    if (units == 1) return ws <= 2 ? 4 : ws <= 4 ? 2 : 1;
+    if (units == 2) return ws <= 2 ? 2 : 1;
+    return 1;
+}
 
 // K_VECS: a row of nvec (1..32) 16-byte vectors is owned by a team of 2^lt lanes
 // (the smallest of 1, 2, 4, 8 that holds it with one vector per lane, else 8),
@@ -73,6 +86,7 @@ static inline int tftq_small_rows_per_wg(int nvec)
     tftq_small_shape(nvec, &lt, &c);
     return (TFTQ_WG >> lt) * (8 / c);
 }
+
 constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
 
 // Rows a workgroup can hold in registers.  The regular kernels keep up to 8

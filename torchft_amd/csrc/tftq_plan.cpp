@@ -93,18 +93,19 @@ static uint8_t pick_reduce_kind(const Seg &s)
     return K_GEN256;
 }
 
-static int rows_per_wg_of(const Seg &s, int st, int esz)
+static int rows_per_wg_of(const Seg &s, int st, int esz, int ws)
 {
     if (s.kind[st] == K_COL1) return 4 * TFTQ_WG;
     if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
     const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
-    return teams;  // one row per team in every stage
+    if (st == ST_R) return teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws);
+    return teams;
 }
 
 // Bytes one workgroup of segment s moves in a stage.
 static double wg_weight(const Seg &s, int st, int esz, int ws)
 {
-    const double rows = (double)rows_per_wg_of(s, st, esz);
+    const double rows = (double)rows_per_wg_of(s, st, esz, ws);
     if (st == ST_R) return rows * (double)s.row_bytes * (ws + 1);
     return rows * ((double)s.n * esz + (double)s.row_bytes);
 }
@@ -279,7 +280,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         s.kind[ST_R] = pick_reduce_kind(s);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
-            const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st, p->esz));
+            const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st, p->esz, ws));
             wgs[i][st] = (int32_t)n;
             wg[st] += n;
             if (wg[st] > INT32_MAX - 4096) {

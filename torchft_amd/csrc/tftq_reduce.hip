@@ -454,6 +454,112 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
     }
 }
 
+// Few peers (ws <= 4): ROWS consecutive rows of one team at once, all loads of
+// all rows issued together, so that a lane has 8 vectors in flight although a
+// row has only ws * UNITS of them.  ws * UNITS * ROWS <= 8.  Rows past the end of
+// the tensor are given the last row and store nothing.  lds: 4 * ROWS floats.
+template <int TEAM, int UNITS, int ROWS, bool GDIV>
+DEV void reduce_rows_at_once(const Seg &s, const KParams &p, int j0, int lane, float *lds)
+{
+    constexpr int PEERS = 8 / (UNITS * ROWS);  // ws <= PEERS
+    const int ndw = (s.row_bytes >> 2) - 1;    // >= 4 here
+    const int ws = p.ws;
+    const int wlane = (int)(threadIdx.x & 63u);
+    const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
+
+    int doff[UNITS];
+    u32 padmask[UNITS];  // as in reduce_rows
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        doff[u] = min(4 * (u * TEAM + lane), ndw - 4);
+        padmask[u] = (doff[u] == ndw - 4 && (s.n & 3)) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+    }
+
+    int64_t off[ROWS];
+    bool valid[ROWS];
+    float raw_scale[ROWS];
+    u32x4 w[ROWS][PEERS][UNITS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        valid[r] = j0 + r < s.slice_rows;
+        off[r] = s.slot_off + (int64_t)min(j0 + r, s.slice_rows - 1) * s.row_bytes;
+        raw_scale[r] = as_f(peer_row(p, speer, off[r])[0]);
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int k = 0; k < PEERS; k++) {
+            GLOBAL const u32 *pv = peer_row(p, min(k, ws - 1), off[r]) + 1;
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) w[r][k][u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + doff[u]));
+        }
+
+    float amax[ROWS];
+    float acc[ROWS][UNITS][16];
+    bool fast[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const float sc = raw_scale[r] == 0.0f ? 1.0f : raw_scale[r];  // padding rows (:419)
+        const DivCoef c = make_div(sc);
+        fast[r] = __builtin_amdgcn_ballot_w64(!c.fast) == 0;  // same in all wavefronts of the team
+#pragma unroll
+        for (int u = 0; u < UNITS; u++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[r][u][e] = 0.0f;
+        amax[r] = 0.0f;
+        if (fast[r]) {
+#pragma unroll
+            for (int k = 0; k < PEERS; k++) {
+                if (k < ws) {
+                    const float pr = bcast_lane(c.r, k), pl = bcast_lane(c.r_lo, k);
+#pragma unroll
+                    for (int u = 0; u < UNITS; u++) {
+                        u32x4 v = w[r][k][u];
+                        v.w &= padmask[u];
+                        accumulate16(acc[r][u], v, pr, pl);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNITS; u++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) amax[r] = fmaxf(amax[r], __builtin_fabsf(acc[r][u][e]));
+        }
+    }
+
+    // row maxima over the team: inside the wavefront, then across the four wavefronts
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) amax[r] = team_max<64>(amax[r], lds);
+    if (TEAM == 256) {
+        const int wave = threadIdx.x >> 6;
+        if (wlane == 0) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) lds[wave * ROWS + r] = amax[r];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < ROWS; r++)
+            amax[r] = fmaxf(fmaxf(lds[r], lds[ROWS + r]), fmaxf(lds[2 * ROWS + r], lds[3 * ROWS + r]));
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        if (fast[r]) {
+            const float s2 = calc_scale(amax_div<GDIV>(amax[r], p));  // :340
+            GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off[r]);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                const u32x4 o = requant16<GDIV>(acc[r][u], s2, p);
+                if (valid[r] && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
+            }
+            if (valid[r] && lane == 0) orow[0] = as_u(s2);  // :375
+        } else if (valid[r]) {
+            reduce_row_slow<TEAM, GDIV>(s, p, j0 + r, lane, lds);  // some peer needs the plain divide
+        }
+    }
+}
+
 // Rows of one column: 8 bytes per row and peer, one plain divide per peer
 // (coefficients for the fast division would cost two), four rows per lane.
 template <bool GDIV>
@@ -491,7 +597,7 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 template <bool INLINE, bool GDIV, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
 {
-    __shared__ float lds[4];
+    __shared__ float lds[16];
     Seg s;
     int vb;
     if (!locate<INLINE, ST_R>(p, inl, s, vb)) return;
@@ -499,9 +605,15 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
     const int tid = threadIdx.x;
     const int ndw = (s.row_bytes >> 2) - 1;
     switch (s.kind[ST_R]) {
-    case K_GEN256: {  // one workgroup per row
-        const int j = blk;
-        if (WIDE && ndw > TFTQ_R_DWORDS && ndw <= TFTQ_R_DWORDS_WIDE && p.ws <= 64) {
+    case K_GEN256: {  // one workgroup per row, or per 2 or 4 rows when the group is small
+        const int rows = tftq_reduce_rows_at_once(K_GEN256, ndw, p.ws);
+        const int j = blk * rows;
+        if (rows == 4) {
+            reduce_rows_at_once<256, 1, 4, GDIV>(s, p, j, tid, lds);
+        } else if (rows == 2) {
+            if (ndw <= 1024) reduce_rows_at_once<256, 1, 2, GDIV>(s, p, j, tid, lds);
+            else reduce_rows_at_once<256, 2, 2, GDIV>(s, p, j, tid, lds);
+        } else if (WIDE && ndw > TFTQ_R_DWORDS && ndw <= TFTQ_R_DWORDS_WIDE && p.ws <= 64) {
             reduce_rows<256, 8, false, GDIV>(s, p, j, tid, lds);
         } else if (ndw > TFTQ_R_DWORDS) {
             if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
@@ -518,10 +630,16 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         }
         break;
     }
-    case K_GEN64: {  // one wavefront per row
-        const int j = blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);
+    case K_GEN64: {  // one wavefront per row, or per 2 or 4 rows when the group is small
+        const int rows = tftq_reduce_rows_at_once(K_GEN64, ndw, p.ws);
+        const int j = (blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6)) * rows;
         if (j >= s.slice_rows) break;  // the whole wavefront leaves
-        if (p.ws > 64) {
+        if (rows == 4) {
+            reduce_rows_at_once<64, 1, 4, GDIV>(s, p, j, tid & 63, lds);
+        } else if (rows == 2) {
+            if (ndw <= 256) reduce_rows_at_once<64, 1, 2, GDIV>(s, p, j, tid & 63, lds);
+            else reduce_rows_at_once<64, 2, 2, GDIV>(s, p, j, tid & 63, lds);
+        } else if (p.ws > 64) {
             if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j, tid & 63, lds);
             else reduce_row<64, 2, GDIV>(s, p, j, tid & 63, lds);
         } else if (ndw <= 256) {
