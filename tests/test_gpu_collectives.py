@@ -167,3 +167,74 @@ def test_world_size_one_is_quantize_dequantize(coll, oracle):
     work.wait()
     torch.cuda.synchronize()
     assert torch.equal(got[0].cpu().view(torch.int16), want[0].view(torch.int16))
+
+
+@pytest.fixture(scope="module")
+def rccl_group_of_one():
+    """A real torch.distributed process group over RCCL (backend "nccl") with this
+    process as its only rank: the work objects, futures and callback threads are
+    ProcessGroupNCCL's own, only the exchange itself is trivial."""
+    import socket
+
+    import torch.distributed as dist
+
+    if not dist.is_nccl_available():
+        pytest.skip("torch.distributed has no nccl (RCCL) backend")
+    assert not dist.is_initialized()
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+    torch.cuda.set_device(0)
+    dist.init_process_group("nccl", init_method=f"tcp://127.0.0.1:{port}", rank=0, world_size=1,
+                            device_id=torch.device("cuda:0"))
+    try:
+        yield dist.distributed_c10d._get_default_group()
+    finally:
+        dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("op", [ReduceOp.SUM, ReduceOp.AVG])
+def test_collectives_over_rccl_group_of_one(coll, oracle, rccl_group_of_one, op):
+    """allreduce_quantized, reduce_scatter_quantized and the managed all-reduce through
+    c10d's ProcessGroup API (alltoall_base, allgather_into_tensor_coalesced, Work,
+    Future.add_done_callback), bytes against the CPU checker."""
+    from torchft_amd.allreduce import allreduce
+
+    pg = rccl_group_of_one
+    g = torch.Generator().manual_seed(5)
+    cpu = [torch.randn(300, 512, generator=g).to(torch.bfloat16),
+           torch.randn(1000, generator=g).to(torch.bfloat16),
+           torch.randn(7, 33, generator=g).to(torch.bfloat16)]
+    want = [t.clone() for t in cpu]
+    packed = oracle.fused_quantize_into_fp8(want, 1)  # 1-D -> [k, 1] in `want`
+    oracle.fused_reduce_fp8(want, packed, 1, 0, op)
+    oracle.fused_dequantize_from_fp8(want, packed, 1)
+
+    stream = torch.cuda.Stream()
+    got = [t.cuda() for t in cpu]
+    work = coll.allreduce_quantized(got, op, pg, stream)
+    work.wait()
+    work.get_future().wait()
+    stream.synchronize()
+    for a, e in zip(got, want):
+        assert torch.equal(a.cpu().reshape(-1).view(torch.int16), e.reshape(-1).view(torch.int16))
+
+    src = [t.cuda() for t in cpu]
+    out, _ = coll.allocate_reduce_scatter_output(src, 1)
+    work = coll.reduce_scatter_quantized(out, src, op, pg, stream)
+    work.wait()
+    work.get_future().wait()
+    stream.synchronize()
+    flat = torch.cat([e.reshape(-1) for e in want])
+    assert torch.equal(out.cpu().view(torch.int16), flat.view(torch.int16))
+
+    # the managed all-reduce: AVG becomes SUM for the collective, then / num_participants
+    x = cpu[0].cuda()
+    w = allreduce(x, pg, num_participants=1, should_quantize=True, reduce_op=op)
+    w.wait()
+    torch.cuda.synchronize()
+    want_sum = [cpu[0].clone()]
+    p = oracle.fused_quantize_into_fp8(want_sum, 1)
+    oracle.fused_reduce_fp8(want_sum, p, 1, 0, ReduceOp.SUM)
+    oracle.fused_dequantize_from_fp8(want_sum, p, 1)
+    assert torch.equal(x.cpu().view(torch.int16), want_sum[0].view(torch.int16))
