@@ -130,6 +130,19 @@ int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_bytes, int r
 int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
                     void *stream);
 
+/*
+ * fused_dequantize_from_fp8 followed by the caller's normalisation of the result,
+ * `tensor /= num_participants` in the continuation of Manager.allreduce
+ * (manager.py:450-452), in one pass over the tensors instead of two.  Writes
+ * cast(float(cast(float(code) / scale)) * post_scale): the value is rounded to
+ * the tensors' dtype as tftq_dequantize stores it, widened again and multiplied
+ * in fp32, which is what torch's division of a GPU tensor by a host scalar
+ * computes with post_scale = (float)(1.0 / divisor).  The bytes equal those of
+ * tftq_dequantize followed by that division.
+ */
+int tftq_dequantize_scaled(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
+                           float post_scale, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -368,6 +368,58 @@ def test_long_rows(q, oracle):
         full_check(q, oracle, peers * 2, 4, ReduceOp.SUM, ranks=[3])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("divisor", [2, 3, 7, 12, 1000, 2.5])
+def test_dequantize_with_division(q, dtype, divisor):
+    """divide_by folds the caller's `tensor /= n` (manager.py:450-452) into the store of
+    the dequantize kernel.  Expected: the plain dequantize followed by torch's own
+    in-place division of each tensor on the GPU, byte for byte; every lane mapping
+    (short and long rows, whole vectors and tails, single columns, strided and
+    misaligned tensors, more than 16 tensors), rows with scales outside the range of
+    the fast division, zero rows and negative zeros."""
+    g = torch.Generator().manual_seed(31)
+    shapes = [(37, 256), (5, 4096), (130,), (3, 14336), (9, 33), (2, 1024), (64, 16), (40, 48), (11, 520),
+              (6, 2100), (3, 9001), (300,), (17, 8), (5, 24), (2, 40000), (1, 1), (4, 100), (8, 64)]
+    cpu = []
+    for sh in shapes:
+        x = torch.randn(sh, generator=g) * 0.3
+        if x.dim() == 2 and x.shape[0] > 2:
+            x[0] *= 1e-30
+            x[1] = 0.0
+            x[2, ::2] = -0.0
+        cpu.append(x.to(dtype))
+    base = torch.randn(50, 300, generator=g).to(dtype)
+    flat = torch.randn(5000, generator=g).to(dtype)
+    for ws, count in ((1, len(cpu)), (4, 9)):  # 20 tensors: device table; 11: in the kernel arguments
+        gbase, gflat = base.cuda(), flat.cuda()
+        src = [t.cuda() for t in cpu[:count]] + [gbase[::2, 1:200:3], gflat[3:3 + 77 * 13].view(77, 13)]
+        packed = q.fused_quantize_into_fp8(list(src), ws)
+
+        def destinations():  # like the sources: the last two strided and misaligned
+            out = [torch.full_like(t, 5.0) for t in src[:count]]
+            b, f = torch.full_like(gbase, 5.0), torch.full_like(gflat, 5.0)
+            return out + [b[::2, 1:200:3], f[3:3 + 77 * 13].view(77, 13)]
+
+        want = destinations()
+        q.fused_dequantize_from_fp8(list(want), packed, ws)
+        for t in want:
+            t /= divisor
+        got = destinations()
+        assert got[-2].stride() == (600, 3) and got[-1].data_ptr() % 16 != 0
+        q.fused_dequantize_from_fp8(list(got), packed, ws, divide_by=divisor)
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            if dtype == torch.float16:
+                # torch's own division of a float16 tensor turns -0 into +0 in the elements
+                # its vectorised loop does not cover (short tensors, tails) and keeps -0
+                # elsewhere; the kernel keeps -0 (IEEE).  Compare with +0 for both.
+                a, b = a.contiguous().clone(), b.contiguous().clone()
+                for t in (a, b):
+                    bits = t.view(torch.int16)
+                    bits[bits == -32768] = 0
+            same_bytes(a, b, f"ws={ws} tensor {i} {tuple(a.shape)}")
+
+
 def test_extreme_scales_and_denormals(q, oracle):
     """Row maxima far outside the range where the fast division applies
     (scale exponent beyond +-64), fp32 denormal inputs, all-zero rows."""

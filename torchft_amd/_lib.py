@@ -39,6 +39,8 @@ SYMBOLS = [
     ("tftq_reduce", _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_int,
                                _c.c_void_p]),
     ("tftq_dequantize", _c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p]),
+    ("tftq_dequantize_scaled", _c.c_int,
+     [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_float, _c.c_void_p]),
 ]
 
 

@@ -10,7 +10,9 @@ which stream, and what is done to the result.
 
 * ``allreduce`` zeroes the tensor of a replica that is not participating, turns
   AVG into SUM for the collective and divides by the number of participants in
-  a continuation of the collective's future (manager.py:419-456).  With
+  a continuation of the collective's future (manager.py:419-456); on the
+  quantized path the division is done by the dequantize kernel as it stores
+  (same bytes, one read and one write of the tensor less).  With
   ``should_quantize`` the list ``[tensor]`` goes to ``allreduce_quantized`` on
   the current stream (manager.py:432-439); a 1-D tensor is quantized as rows of
   one column (quantization.py:487-488), 8 packed bytes per element.
@@ -106,10 +108,14 @@ def allreduce(
     is_participating: bool = True,
     should_quantize: bool = False,
     reduce_op: ReduceOp = ReduceOp.AVG,
+    fold_normalization: bool = True,
 ):
     """
     All-reduce ``tensor`` in place over ``process_group`` and scale it by
     ``1 / num_participants`` when ``reduce_op`` is AVG (manager.py:386-456).
+    With ``should_quantize`` the scaling is part of the dequantize kernel unless
+    ``fold_normalization`` is False (then it is a separate in-place division in
+    the continuation, as in the reference); the resulting bytes are the same.
 
     Returns a work whose future completes with the tensor.  The result is in
     ``tensor`` once the work has been waited on, in stream order of the stream
@@ -124,8 +130,14 @@ def allreduce(
             raise ValueError("average reduce op is only supported for floating point tensors")
         pg_reduce_op = ReduceOp.SUM  # manager.py:422-429
 
+    normalized = False
     if should_quantize:
-        work = allreduce_quantized([tensor], pg_reduce_op, process_group, torch.cuda.current_stream())
+        # the division by the number of participants (manager.py:450-452) happens in the
+        # dequantize kernel: same bytes, one pass over the tensor less
+        divide_by = num_participants if reduce_op == ReduceOp.AVG and fold_normalization else None
+        normalized = divide_by is not None
+        work = allreduce_quantized([tensor], pg_reduce_op, process_group, torch.cuda.current_stream(),
+                                   divide_by=divide_by)
     else:
         opts = AllreduceOptions()
         opts.reduceOp = pg_reduce_op
@@ -134,7 +146,7 @@ def allreduce(
     chained = _ChainedWork(work, tensor)
 
     def normalize(value: torch.Tensor) -> torch.Tensor:
-        if reduce_op == ReduceOp.AVG:
+        if reduce_op == ReduceOp.AVG and not normalized:
             value /= num_participants  # manager.py:450-452
         return value
 

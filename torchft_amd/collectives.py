@@ -183,12 +183,19 @@ def allreduce_quantized(
     opts: AllreduceOptions | ReduceOp,
     process_group: Any,
     sync_stream: cuda.Stream | None = None,
+    *,
+    divide_by: float | None = None,
 ):
     """
     Quantized all-reduce of ``tensors`` in place.  Only AVG and SUM are
     supported (``NotImplementedError`` otherwise).  Returns the all-gather work;
     the tensors hold the result once the work's future has run its callbacks
     and ``sync_stream`` has been waited on (collectives.py:297-415).
+
+    ``divide_by`` (no counterpart in the reference's function): the tensors are
+    left as if each had then been divided by that Python number on the GPU, as
+    ``Manager.allreduce`` does with the number of participants
+    (manager.py:450-452), at no extra pass over them.
     """
     ex = _begin(opts, AllreduceOptions, "allreduce", process_group, sync_stream)
     ws, rank = ex.world_size, ex.rank
@@ -202,5 +209,5 @@ def allreduce_quantized(
         # the reduced slots of all ranks land in the first buffer
         work = ex.gather_slots(packed, received)
         work.wait()  # a stream dependency with RCCL, not a host block
-        ex.finish_on_stream(work, lambda: _q._dequantize(plan, device, packed))
+        ex.finish_on_stream(work, lambda: _q._dequantize(plan, device, packed, divide_by))
     return work

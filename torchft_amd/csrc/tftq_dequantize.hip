@@ -18,9 +18,19 @@ DEV bool rows_fill_lines(const Seg &s)
     return ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ) | (uint64_t)((int64_t)s.n * Elem<T>::ESZ)) & 63u) == 0;
 }
 
+// The value that is stored: the quotient, or in the scaled variant (POST) the
+// quotient as it reads back from the tensor's dtype, times post_scale: the
+// caller's `tensor /= num_participants` (manager.py:450-452) without a second
+// pass over the tensor.
+template <typename T, bool POST>
+DEV float fin(float v, const KParams &p)
+{
+    return POST ? Elem<T>::rounded(v) * p.post_scale : v;
+}
+
 // Any strides; also the path of rows whose scale is outside the range of the
 // fast exact division (plain IEEE divide, one element per lane and step).
-template <typename T, int TEAM>
+template <typename T, int TEAM, bool POST>
 DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
 {
     if (row >= s.m) return;
@@ -31,13 +41,13 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
     if (c.fast) {
         for (int col = lane; col < s.n; col += TEAM) {
             const float f = __builtin_amdgcn_cvt_f32_fp8((int)in[4 + col], 0);
-            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, div_fast_signed(f, c.r, c.r_lo));
+            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p));
         }
     } else {
 #pragma nounroll
         for (int col = lane; col < s.n; col += TEAM) {
             const float f = __builtin_amdgcn_cvt_f32_fp8((int)in[4 + col], 0);
-            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, f / c.s);
+            Elem<T>::store(base, r0 + (int64_t)col * s.col_stride, fin<T, POST>(f / c.s, p));
         }
     }
 }
@@ -45,14 +55,14 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
 // Contiguous, 16-byte aligned rows.  Four vectors per lane and step; their loads
 // are issued together without a branch (lanes past the end re-read the last
 // vector and do not store).
-template <typename T, int TEAM, bool NT, int DV>
+template <typename T, int TEAM, bool NT, int DV, bool POST>
 DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
 {
     if (row >= s.m) return;
     GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
     const DivCoef c = make_div(as_f(in[0]));
     if (!c.fast) {  // same for all lanes of the team
-        dequantize_gen<T, TEAM>(s, p, row, lane);
+        dequantize_gen<T, TEAM, POST>(s, p, row, lane);
         return;
     }
     constexpr int EPV = Elem<T>::EPV;
@@ -61,7 +71,7 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
     // the few columns after the last whole vector, one element per lane
     for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
         const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
-        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, div_fast_signed(f, c.r, c.r_lo));
+        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p));
     }
     for (int base = 0; base < nvec; base += DV * TEAM) {
         u32x2 w[DV];
@@ -82,11 +92,11 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
             float f[4];
             unpack_fp8x4(w[k].x, f);
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], c.r, c.r_lo);
+            for (int e = 0; e < 4; e++) o[e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
             if constexpr (EPV == 8) {
                 unpack_fp8x4(w[k].y, f);
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(f[e], c.r, c.r_lo);
+                for (int e = 0; e < 4; e++) o[4 + e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
             }
             if (idx < nvec) {
                 if (NT) STORE_STREAM(Elem<T>::pack(o), out + idx);
@@ -96,7 +106,7 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
-template <typename T, int TEAM>
+template <typename T, int TEAM, bool POST>
 DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
 {
     // same branch for the whole workgroup
@@ -104,16 +114,16 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
     // on 4096-column bf16 rows), 4 for shorter rows, whose lanes would mostly load duplicates
     const bool few = s.n / Elem<T>::EPV <= 4 * TEAM;
     if (rows_fill_lines<T>(s)) {
-        if (few) dequantize_vec_nt<T, TEAM, true, 4>(s, p, row, lane);
-        else dequantize_vec_nt<T, TEAM, true, 8>(s, p, row, lane);
+        if (few) dequantize_vec_nt<T, TEAM, true, 4, POST>(s, p, row, lane);
+        else dequantize_vec_nt<T, TEAM, true, 8, POST>(s, p, row, lane);
     } else {
-        if (few) dequantize_vec_nt<T, TEAM, false, 4>(s, p, row, lane);
-        else dequantize_vec_nt<T, TEAM, false, 8>(s, p, row, lane);
+        if (few) dequantize_vec_nt<T, TEAM, false, 4, POST>(s, p, row, lane);
+        else dequantize_vec_nt<T, TEAM, false, 8, POST>(s, p, row, lane);
     }
 }
 
 // Rows of one column: one plain divide per row, four rows per lane.
-template <typename T>
+template <typename T, bool POST>
 DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 {
     u32x2 w[4];
@@ -126,13 +136,13 @@ DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
     for (int k = 0; k < 4; k++) {
         const int row = row0 + k * TFTQ_WG + tid;
         const float f = __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0);
-        if (row < s.m) Elem<T>::store(s.ptr, (int64_t)row * s.row_stride, f / as_f(w[k].x));  // no zero guard (:239)
+        if (row < s.m) Elem<T>::store(s.ptr, (int64_t)row * s.row_stride, fin<T, POST>(f / as_f(w[k].x), p));  // no zero guard (:239)
     }
 }
 
 // K_VECS in dequantize: same shape as quantize_small, 8 vectors of codes and their
 // rows' scales in flight per lane.
-template <typename T, int C, bool NT>
+template <typename T, int C, bool NT, bool POST>
 DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
 {
     constexpr int EPV = Elem<T>::EPV;
@@ -176,17 +186,17 @@ DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, co
             unpack_fp8x4(w[r][k].y, g);
             if (fast) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = div_fast_signed(f[e], c.r, c.r_lo);
+                for (int e = 0; e < 4; e++) o[e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
                 if constexpr (EPV == 8) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[4 + e] = div_fast_signed(g[e], c.r, c.r_lo);
+                    for (int e = 0; e < 4; e++) o[4 + e] = fin<T, POST>(div_fast_signed(g[e], c.r, c.r_lo), p);
                 }
             } else {
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = f[e] / sc[r];  // :250-252
+                for (int e = 0; e < 4; e++) o[e] = fin<T, POST>(f[e] / sc[r], p);  // :250-252
                 if constexpr (EPV == 8) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[4 + e] = g[e] / sc[r];
+                    for (int e = 0; e < 4; e++) o[4 + e] = fin<T, POST>(g[e] / sc[r], p);
                 }
             }
             const int vec = k * h.team + h.l;
@@ -198,24 +208,24 @@ DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, co
     }
 }
 
-template <typename T>
+template <typename T, bool POST>
 DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid)
 {
     const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
     if (rows_fill_lines<T>(s)) {
-        if (h.c == 1) dequantize_small_c<T, 1, true>(s, p, blk, tid, h);
-        else if (h.c == 2) dequantize_small_c<T, 2, true>(s, p, blk, tid, h);
-        else if (h.c == 3) dequantize_small_c<T, 3, true>(s, p, blk, tid, h);
-        else dequantize_small_c<T, 4, true>(s, p, blk, tid, h);
+        if (h.c == 1) dequantize_small_c<T, 1, true, POST>(s, p, blk, tid, h);
+        else if (h.c == 2) dequantize_small_c<T, 2, true, POST>(s, p, blk, tid, h);
+        else if (h.c == 3) dequantize_small_c<T, 3, true, POST>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 4, true, POST>(s, p, blk, tid, h);
     } else {
-        if (h.c == 1) dequantize_small_c<T, 1, false>(s, p, blk, tid, h);
-        else if (h.c == 2) dequantize_small_c<T, 2, false>(s, p, blk, tid, h);
-        else if (h.c == 3) dequantize_small_c<T, 3, false>(s, p, blk, tid, h);
-        else dequantize_small_c<T, 4, false>(s, p, blk, tid, h);
+        if (h.c == 1) dequantize_small_c<T, 1, false, POST>(s, p, blk, tid, h);
+        else if (h.c == 2) dequantize_small_c<T, 2, false, POST>(s, p, blk, tid, h);
+        else if (h.c == 3) dequantize_small_c<T, 3, false, POST>(s, p, blk, tid, h);
+        else dequantize_small_c<T, 4, false, POST>(s, p, blk, tid, h);
     }
 }
 
-template <typename T, bool INLINE>
+template <typename T, bool INLINE, bool POST>
 __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const InlineTable inl)
 {
     Seg s;
@@ -224,53 +234,67 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
     const int blk = vb - s.wg_begin[ST_D];
     const int tid = threadIdx.x;
     switch (s.kind[ST_D]) {
-    case K_VEC256: dequantize_vec<T, 256>(s, p, blk, tid); break;
+    case K_VEC256: dequantize_vec<T, 256, POST>(s, p, blk, tid); break;
     case K_VEC64:
-        dequantize_vec<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
+        dequantize_vec<T, 64, POST>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;
-    case K_VEC32: dequantize_vec<T, 32>(s, p, blk * 8 + (tid >> 5), tid & 31); break;
-    case K_VEC16: dequantize_vec<T, 16>(s, p, blk * 16 + (tid >> 4), tid & 15); break;
-    case K_VEC8: dequantize_vec<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
+    case K_VEC32: dequantize_vec<T, 32, POST>(s, p, blk * 8 + (tid >> 5), tid & 31); break;
+    case K_VEC16: dequantize_vec<T, 16, POST>(s, p, blk * 16 + (tid >> 4), tid & 15); break;
+    case K_VEC8: dequantize_vec<T, 8, POST>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN64:
-        dequantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
+        dequantize_gen<T, 64, POST>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;
-    case K_GEN8: dequantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
-    case K_GEN1: dequantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
+    case K_GEN8: dequantize_gen<T, 8, POST>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
+    case K_GEN1: dequantize_gen<T, 1, POST>(s, p, blk * 256 + tid, 0); break;
     case K_COL1:
-        if (s.m > 0) dequantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid);
+        if (s.m > 0) dequantize_col1<T, POST>(s, p, blk * 4 * TFTQ_WG, tid);
         break;
-    case K_VECS: dequantize_small<T>(s, p, blk, tid); break;
+    case K_VECS: dequantize_small<T, POST>(s, p, blk, tid); break;
     default: break;
     }
 }
 
-template <typename T>
+template <typename T, bool POST>
 static int launch_d(const KParams &kp, const InlineTable &inl, bool use_inline, hipStream_t st)
 {
     if (use_inline)
-        hipLaunchKernelGGL((k_dequantize<T, true>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
+        hipLaunchKernelGGL((k_dequantize<T, true, POST>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
     else
-        hipLaunchKernelGGL((k_dequantize<T, false>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
+        hipLaunchKernelGGL((k_dequantize<T, false, POST>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
     return (int)hipGetLastError();
 }
 
-extern "C" int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
-                               void *stream)
+template <bool POST>
+static int dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes, float post_scale,
+                      void *stream)
 {
     KParams kp;
     InlineTable inl = {};
     bool use_inline;
     int rc = fill_params(plan, ST_D, (void *)packed, packed_bytes, &kp, &inl, &use_inline);
     if (rc) return rc;
+    kp.post_scale = post_scale;
     for (int i = 0; i < plan->nseg; i++)
         if (plan->segs[(size_t)i].ptr == 0 && plan->segs[(size_t)i].m > 0 && plan->segs[(size_t)i].n > 0)
             return TFTQ_E_ARG;
     if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
     switch (plan->dtype) {
-    case TFTQ_F32: return launch_d<float>(kp, inl, use_inline, st);
-    case TFTQ_F16: return launch_d<f16_tag>(kp, inl, use_inline, st);
-    case TFTQ_BF16: return launch_d<bf16_tag>(kp, inl, use_inline, st);
+    case TFTQ_F32: return launch_d<float, POST>(kp, inl, use_inline, st);
+    case TFTQ_F16: return launch_d<f16_tag, POST>(kp, inl, use_inline, st);
+    case TFTQ_BF16: return launch_d<bf16_tag, POST>(kp, inl, use_inline, st);
     default: return TFTQ_E_DTYPE;
     }
+}
+
+extern "C" int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
+                               void *stream)
+{
+    return dequantize<false>(plan, packed, packed_bytes, 1.0f, stream);
+}
+
+extern "C" int tftq_dequantize_scaled(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
+                                      float post_scale, void *stream)
+{
+    return dequantize<true>(plan, packed, packed_bytes, post_scale, stream);
 }

@@ -207,6 +207,7 @@ template <> struct Elem<float> {
     }
     DEV static float load(uint64_t base, int64_t idx) { return as_global<const float>(base)[idx]; }
     DEV static void store(uint64_t base, int64_t idx, float v) { as_global<float>(base)[idx] = v; }
+    DEV static float rounded(float v) { return v; }  // v as a stored element reads back
 };
 
 template <> struct Elem<bf16_tag> {
@@ -238,6 +239,7 @@ template <> struct Elem<bf16_tag> {
     {
         as_global<uint16_t>(base)[idx] = (uint16_t)(pack2(v, 0.0f) & 0xFFFFu);
     }
+    DEV static float rounded(float v) { return as_f(pack2(v, 0.0f) << 16); }
 };
 
 template <> struct Elem<f16_tag> {
@@ -282,6 +284,7 @@ template <> struct Elem<f16_tag> {
     {
         as_global<_Float16>(base)[idx] = (_Float16)opaque(v);
     }
+    DEV static float rounded(float v) { return (float)(_Float16)opaque(v); }
 };
 
 // ---------------------------------------------------------------------------
@@ -446,6 +449,7 @@ static inline int fill_params(const tftq_plan *plan, int stage, void *packed, in
     kp->div_mode = 0;
     kp->div = 1.0f;
     kp->inv_div = 1.0f;
+    kp->post_scale = 1.0f;
     if (*use_inline)
         for (int i = 0; i < plan->nseg; i++) inl->s[i] = plan->segs[(size_t)i];
     return 0;

@@ -185,4 +185,5 @@ struct KParams {
     int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG general
     float div;          // reduce: 1.0 or float(ws)
     float inv_div;      // reduce: exact reciprocal when div_mode == 1
+    float post_scale;   // dequantize: factor applied to the rounded result (scaled variant only)
 };

@@ -236,12 +236,21 @@ def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
         _keep_table(plan, device)
 
 
-def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor) -> None:
+def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor,
+                divide_by: float | None = None) -> None:
     _check_packed(output, plan, device)
     with _on_device(device):
-        _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                         plan.output_size, _stream_ptr(device)),
-               "tftq_dequantize")
+        if divide_by is None:
+            _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                             plan.output_size, _stream_ptr(device)),
+                   "tftq_dequantize")
+        else:
+            # torch divides a GPU tensor by a host scalar as a multiplication by the
+            # reciprocal, computed in double and rounded to fp32
+            _check(plan._lib.tftq_dequantize_scaled(plan.handle, ctypes.c_void_p(output.data_ptr()),
+                                                    plan.output_size, 1.0 / divide_by,
+                                                    _stream_ptr(device)),
+                   "tftq_dequantize_scaled")
         _keep_table(plan, device)
 
 
@@ -265,15 +274,21 @@ def fused_quantize_into_fp8(
 
 
 def fused_dequantize_from_fp8(
-    inputs: list[torch.Tensor], output: torch.Tensor, all_reduce_group_size: int
+    inputs: list[torch.Tensor], output: torch.Tensor, all_reduce_group_size: int,
+    *, divide_by: float | None = None,
 ) -> None:
     """
     Dequantizes the packed tensor ``output`` into ``inputs`` in place
     (quantization.py:591-635).  The tensors must have the shapes that were
     quantized.
+
+    ``divide_by`` (no counterpart in the reference's function) folds the caller's
+    ``tensor /= divide_by`` (manager.py:450-452) into the same pass: the tensors end
+    up with the bytes that dequantizing and then dividing each of them by that
+    Python number on the GPU gives.
     """
     plan, device = _prepare(inputs, all_reduce_group_size)
-    _dequantize(plan, device, output)
+    _dequantize(plan, device, output, divide_by)
 
 
 def fused_reduce_fp8(
