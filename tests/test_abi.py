@@ -96,6 +96,17 @@ def test_plan_errors():
     assert b"Output size does not match" == _lib.load().tftq_strerror(-4)
 
 
+def test_plan_rejects_grids_the_hardware_cannot_launch():
+    """A grid has fewer than 2^32 threads = 2^24 workgroups of 256.  Rows of 600 fp32
+    columns are quantized by 32 lanes each, eight to a workgroup."""
+    rc, h = _plan(0, [(8 * (2 ** 24 - 64), 600)], [(600, 1)], 1)
+    assert rc == 0
+    _lib.load().tftq_plan_destroy(h)
+    assert _plan(0, [(8 * 2 ** 24 + 64, 600)], [(600, 1)], 1)[0] == -3
+    # the same rows spread over 20 tensors (device table): rejected as well
+    assert _plan(0, [((8 * 2 ** 24) // 20 + 64, 600)] * 20, [(600, 1)] * 20, 1)[0] == -3
+
+
 def test_host_wrapper_validation_messages():
     """Same assertion texts as torchft/quantization.py:463-489."""
     from torchft_amd import quantization as q

@@ -305,6 +305,14 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         delete p;
         return TFTQ_E_NOMEM;
     }
+    // a grid has fewer than 2^32 threads
+    for (int st = 0; st < 3; st++) {
+        const int64_t per_xcd = p->nseg <= TFTQ_N_INLINE ? p->dealt_per_xcd[st] : p->index[st].per_xcd;
+        if (8 * per_xcd * TFTQ_WG > (int64_t)UINT32_MAX) {
+            delete p;
+            return TFTQ_E_SHAPE;
+        }
+    }
     *out = p;
     return 0;
 }
