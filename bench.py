@@ -291,7 +291,7 @@ def main() -> int:
     # The roofline entry is for the kernel that takes the largest share of the step.
     # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE (x2.000,
     # calibrated on a 256 MiB copy) + WRITE_SIZE (x1.000); profiles/cfg3_bf16_ws8_hbm_traffic.md
-    measured_traffic = {"quantize": 655147000, "reduce": 246596000, "dequantize": 661426000}
+    measured_traffic = {"quantize": 655142000, "reduce": 246760000, "dequantize": 661483000}
     achieved = ab[dominant] / (dominant_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "k_" + dominant, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
