@@ -110,7 +110,7 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
             const int64_t m_pad = (int64_t)s.slice_rows * ws;
             const int64_t rows = st == ST_Q ? m_pad : st == ST_R ? s.slice_rows : s.m;
             int per_wg;
-            if (s.kind[st] == K_COL1) per_wg = 4 * TFTQ_WG;
+            if (s.kind[st] == K_COL1) per_wg = tftq_col1_rows_per_wg(st);
             else if (s.kind[st] == K_VECS) per_wg = tftq_small_rows_per_wg(s.n / (dtype == TFTQ_F32 ? 4 : 8));
             else {
                 const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);

@@ -122,21 +122,66 @@ DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
-// Rows of one column: one plain divide per row, four rows per lane.
+// Rows of one column: one plain divide per row.  Any element stride: four rows
+// per lane, interleaved.
 template <typename T, bool POST>
-DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+DEV void dequantize_col1_strided(const Seg &s, const KParams &p, int row0, int tid)
 {
+    const float inv = 1.0f / (float)s.slice_rows;
     u32x2 w[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int row = min(row0 + k * TFTQ_WG + tid, s.m - 1);
-        w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)as_global<const u32>(p.packed + row_addr(s, p.slot_size, row)));
+        w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, row, inv)));
     }
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int row = row0 + k * TFTQ_WG + tid;
         const float f = __builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0);
         if (row < s.m) Elem<T>::store(s.ptr, (int64_t)row * s.row_stride, fin<T, POST>(f / as_f(w[k].x), p));  // no zero guard (:239)
+    }
+}
+
+// Contiguous elements: a lane takes TFTQ_COL1_PAIRS_D pairs of neighbouring rows, reads the
+// two packed rows of a pair with one 16-byte load and writes the two elements
+// with one store (the mapping of quantize_col1).
+template <typename T, bool POST>
+DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+{
+    if (s.row_stride != 1) {  // same for the whole workgroup
+#pragma nounroll
+        for (int r = 0; r < 2 * TFTQ_COL1_PAIRS_D * TFTQ_WG && row0 + r < s.m; r += 4 * TFTQ_WG)
+            dequantize_col1_strided<T, POST>(s, p, row0 + r, tid);
+        return;
+    }
+    const float inv = 1.0f / (float)s.slice_rows;
+    u32x4 w[TFTQ_COL1_PAIRS_D];
+#pragma unroll
+    for (int k = 0; k < TFTQ_COL1_PAIRS_D; k++) {
+        const int row = min(row0 + 2 * (k * TFTQ_WG + tid), s.m - 1);
+        int slot = (int)((float)row * inv);  // off by at most one
+        int j = row - slot * s.slice_rows;
+        if (j < 0) { --slot; j += s.slice_rows; }
+        if (j >= s.slice_rows) { ++slot; j -= s.slice_rows; }
+        GLOBAL const u32 *src = as_global<const u32>(p.packed + (int64_t)slot * p.slot_size + s.slot_off + (int64_t)j * 8);
+        if (j + 1 < s.slice_rows) {  // the next row follows in the same slot
+            w[k] = LOAD_STREAM((GLOBAL const u32x4_a4 *)src);
+        } else {
+            const u32x2 a = LOAD_STREAM((GLOBAL const u32x2_a4 *)src);
+            u32x2 b = {0x3F800000u, 0u};
+            if (row + 1 < s.m)
+                b = LOAD_STREAM((GLOBAL const u32x2_a4 *)as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, row + 1, inv)));
+            w[k] = u32x4{a.x, a.y, b.x, b.y};
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < TFTQ_COL1_PAIRS_D; k++) {
+        const int row = row0 + 2 * (k * TFTQ_WG + tid);
+        // no zero guard (:239)
+        const float a = fin<T, POST>(__builtin_amdgcn_cvt_f32_fp8((int)w[k].y, 0) / as_f(w[k].x), p);
+        const float b = fin<T, POST>(__builtin_amdgcn_cvt_f32_fp8((int)w[k].w, 0) / as_f(w[k].z), p);
+        if (row + 1 < s.m) Elem<T>::store2(s.ptr, row, a, b);
+        else if (row < s.m) Elem<T>::store(s.ptr, row, a);
     }
 }
 
@@ -247,7 +292,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
     case K_GEN8: dequantize_gen<T, 8, POST>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: dequantize_gen<T, 1, POST>(s, p, blk * 256 + tid, 0); break;
     case K_COL1:
-        if (s.m > 0) dequantize_col1<T, POST>(s, p, blk * 4 * TFTQ_WG, tid);
+        if (s.m > 0) dequantize_col1<T, POST>(s, p, blk * tftq_col1_rows_per_wg(ST_D), tid);
         break;
     case K_VECS: dequantize_small<T, POST>(s, p, blk, tid); break;
     default: break;

@@ -47,6 +47,8 @@ typedef u32 u32x2 __attribute__((ext_vector_type(2)));
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x2 u32x2_a4 __attribute__((aligned(4)));
 typedef u32x4 u32x4_a2 __attribute__((aligned(2)));  // tensor rows: aligned to the element only
+typedef u32 u32_a2 __attribute__((aligned(2)));
+typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -208,6 +210,18 @@ template <> struct Elem<float> {
     DEV static float load(uint64_t base, int64_t idx) { return as_global<const float>(base)[idx]; }
     DEV static void store(uint64_t base, int64_t idx, float v) { as_global<float>(base)[idx] = v; }
     DEV static float rounded(float v) { return v; }  // v as a stored element reads back
+    // elements idx and idx + 1 with one access
+    DEV static void load2(uint64_t base, int64_t idx, float &a, float &b)
+    {
+        const u32x2 w = LOAD_STREAM((GLOBAL const u32x2_a4 *)(as_global<const float>(base) + idx));
+        a = as_f(w.x);
+        b = as_f(w.y);
+    }
+    DEV static void store2(uint64_t base, int64_t idx, float a, float b)
+    {
+        const u32x2 w = {as_u(a), as_u(b)};
+        *(GLOBAL u32x2_a4 *)(as_global<float>(base) + idx) = w;
+    }
 };
 
 template <> struct Elem<bf16_tag> {
@@ -240,6 +254,16 @@ template <> struct Elem<bf16_tag> {
         as_global<uint16_t>(base)[idx] = (uint16_t)(pack2(v, 0.0f) & 0xFFFFu);
     }
     DEV static float rounded(float v) { return as_f(pack2(v, 0.0f) << 16); }
+    DEV static void load2(uint64_t base, int64_t idx, float &a, float &b)
+    {
+        const u32 w = LOAD_STREAM((GLOBAL const u32_a2 *)(as_global<const uint16_t>(base) + idx));
+        a = as_f(w << 16);
+        b = as_f(w & 0xFFFF0000u);
+    }
+    DEV static void store2(uint64_t base, int64_t idx, float a, float b)
+    {
+        *(GLOBAL u32_a2 *)(as_global<uint16_t>(base) + idx) = pack2(a, b);
+    }
 };
 
 template <> struct Elem<f16_tag> {
@@ -285,6 +309,14 @@ template <> struct Elem<f16_tag> {
         as_global<_Float16>(base)[idx] = (_Float16)opaque(v);
     }
     DEV static float rounded(float v) { return (float)(_Float16)opaque(v); }
+    DEV static void load2(uint64_t base, int64_t idx, float &a, float &b)
+    {
+        unpack2(LOAD_STREAM((GLOBAL const u32_a2 *)(as_global<const uint16_t>(base) + idx)), a, b);
+    }
+    DEV static void store2(uint64_t base, int64_t idx, float a, float b)
+    {
+        *(GLOBAL u32_a2 *)(as_global<uint16_t>(base) + idx) = pack2(a, b);
+    }
 };
 
 // ---------------------------------------------------------------------------

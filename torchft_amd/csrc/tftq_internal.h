@@ -87,6 +87,20 @@ static inline int tftq_small_rows_per_wg(int nvec)
     return (TFTQ_WG >> lt) * (8 / c);
 }
 
+// K_COL1, rows of one column.  Quantize and dequantize: a lane takes a few pairs of
+// neighbouring rows and issues all its loads together.  Measured on 64 Mi rows,
+// 2 / 4 / 8 pairs per lane: quantize bf16 158 / 143 / 147 us (with 2 pairs a workgroup
+// has only 2 KB of input in flight and waits for it), fp32 137 / 136 / 155 us;
+// dequantize bf16 118 / 117 / 122 us, fp32 131 / 140 / 147 us.
+// Reduce: four rows per lane and peer.
+constexpr int TFTQ_COL1_PAIRS_Q = 4, TFTQ_COL1_PAIRS_D = 2;
+TFTQ_HD static inline int tftq_col1_rows_per_wg(int stage)
+{
+    return stage == ST_Q ? 2 * TFTQ_COL1_PAIRS_Q * TFTQ_WG
+         : stage == ST_D ? 2 * TFTQ_COL1_PAIRS_D * TFTQ_WG
+                         : 4 * TFTQ_WG;
+}
+
 constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
 
 // Rows a workgroup can hold in registers.  The regular kernels keep up to 8

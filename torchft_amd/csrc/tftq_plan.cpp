@@ -95,7 +95,7 @@ static uint8_t pick_reduce_kind(const Seg &s)
 
 static int rows_per_wg_of(const Seg &s, int st, int esz, int ws)
 {
-    if (s.kind[st] == K_COL1) return 4 * TFTQ_WG;
+    if (s.kind[st] == K_COL1) return tftq_col1_rows_per_wg(st);
     if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
     const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
     if (st == ST_R) return teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws);

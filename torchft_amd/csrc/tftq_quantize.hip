@@ -198,12 +198,24 @@ DEV void quantize_gen(const Seg &s, const KParams &p, int row, int lane)
 
 // Rows of one column (1-D tensors, quantization.py:487-488): a row is its own
 // maximum, so the code is +-448 (or 0) and all information is in the scale.
-// Four rows per lane, interleaved so that every load and every 8-byte
+// [scale, code] of one row
+DEV u32x2 quantize_one(float x)
+{
+    // maximum with 0 as for longer rows: a NaN element is ignored (:131-143)
+    const float sc = calc_scale(fmaxf(0.0f, __builtin_fabsf(x)));
+    u32x2 o;
+    o.x = as_u(sc);
+    o.y = pack_fp8x4(x * sc, 0.0f, 0.0f, 0.0f) & 0xFFu;
+    return o;
+}
+
+// Any element stride: four rows per lane, interleaved so that every 8-byte
 // [scale, code] store of a wavefront is contiguous.
 template <typename T>
-DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+DEV void quantize_col1_strided(const Seg &s, const KParams &p, int row0, int tid)
 {
     const int m_pad = s.slice_rows * p.ws;
+    const float inv = 1.0f / (float)s.slice_rows;
     float x[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
@@ -215,13 +227,55 @@ DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
         const int row = row0 + k * TFTQ_WG + tid;
         if (row < m_pad) {
             u32x2 o = {0u, 0u};  // padding rows stay zero
-            if (row < s.m) {
-                // maximum with 0 as for longer rows: a NaN element is ignored (:131-143)
-                const float sc = calc_scale(fmaxf(0.0f, __builtin_fabsf(x[k])));
-                o.x = as_u(sc);
-                o.y = pack_fp8x4(x[k] * sc, 0.0f, 0.0f, 0.0f) & 0xFFu;
-            }
-            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + row_addr(s, p.slot_size, row)) = o;
+            if (row < s.m) o = quantize_one(x[k]);
+            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row, inv)) = o;
+        }
+    }
+}
+
+// Contiguous elements: a lane takes TFTQ_COL1_PAIRS_Q pairs of neighbouring rows, so that it
+// reads two elements with one load (a wavefront reads 256 or 512 contiguous
+// bytes per load even for 2-byte elements) and writes their two packed rows
+// with one 16-byte streaming store (a wavefront writes 1 KB of whole lines).
+// A pair that straddles the end of a slot or of the tensor is stored row by row.
+template <typename T>
+DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
+{
+    if (s.row_stride != 1) {  // same for the whole workgroup
+#pragma nounroll
+        for (int r = 0; r < 2 * TFTQ_COL1_PAIRS_Q * TFTQ_WG && row0 + r < s.slice_rows * p.ws; r += 4 * TFTQ_WG)
+            quantize_col1_strided<T>(s, p, row0 + r, tid);
+        return;
+    }
+    const int m_pad = s.slice_rows * p.ws;
+    const float inv = 1.0f / (float)s.slice_rows;
+    float x[TFTQ_COL1_PAIRS_Q][2];
+#pragma unroll
+    for (int k = 0; k < TFTQ_COL1_PAIRS_Q; k++) {
+        const int row = row0 + 2 * (k * TFTQ_WG + tid);
+        x[k][0] = x[k][1] = 0.0f;
+        if (row + 1 < s.m) Elem<T>::load2(s.ptr, row, x[k][0], x[k][1]);
+        else if (row < s.m) x[k][0] = Elem<T>::load(s.ptr, row);
+    }
+#pragma unroll
+    for (int k = 0; k < TFTQ_COL1_PAIRS_Q; k++) {
+        const int row = row0 + 2 * (k * TFTQ_WG + tid);
+        if (row >= m_pad) continue;
+        u32x2 a = {0u, 0u}, b = {0u, 0u};  // padding rows stay zero
+        if (row < s.m) a = quantize_one(x[k][0]);
+        if (row + 1 < s.m) b = quantize_one(x[k][1]);
+        int slot = (int)((float)row * inv);  // off by at most one
+        int j = row - slot * s.slice_rows;
+        if (j < 0) { --slot; j += s.slice_rows; }
+        if (j >= s.slice_rows) { ++slot; j -= s.slice_rows; }
+        GLOBAL u32 *dst = as_global<u32>(p.packed + (int64_t)slot * p.slot_size + s.slot_off + (int64_t)j * 8);
+        if (j + 1 < s.slice_rows) {  // the next row follows in the same slot (and row + 1 < m_pad)
+            const u32x4 o = {a.x, a.y, b.x, b.y};
+            STORE_STREAM(o, (GLOBAL u32x4_a4 *)dst);
+        } else {
+            *(GLOBAL u32x2_a4 *)dst = a;
+            if (row + 1 < m_pad)
+                *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row + 1, inv)) = b;
         }
     }
 }
@@ -302,7 +356,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
         break;
     case K_GEN8: quantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: quantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
-    case K_COL1: quantize_col1<T>(s, p, blk * 4 * TFTQ_WG, tid); break;
+    case K_COL1: quantize_col1<T>(s, p, blk * tftq_col1_rows_per_wg(ST_Q), tid); break;
     case K_VECS: quantize_small<T>(s, p, blk, tid); break;
     default: break;
     }

@@ -672,7 +672,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         else if (ndw <= 8) reduce_row<1, 2, GDIV>(s, p, blk * 256 + tid, 0, lds);
         else reduce_row<1, 4, GDIV>(s, p, blk * 256 + tid, 0, lds);
         break;
-    case K_COL1: reduce_col1<GDIV>(s, p, blk * 4 * TFTQ_WG, tid); break;
+    case K_COL1: reduce_col1<GDIV>(s, p, blk * tftq_col1_rows_per_wg(ST_R), tid); break;
     default: break;
     }
 }
