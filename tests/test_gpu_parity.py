@@ -369,6 +369,50 @@ def test_long_rows(q, oracle):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("ws", [1, 2, 3, 8])
+def test_single_column_tensors(q, oracle, dtype, ws):
+    """1-D tensors (rows of one column): lengths around the rows a workgroup takes in each
+    stage, odd lengths and odd rows per slot (a lane's pair of rows then straddles two
+    slots or the end of the tensor), starts that are not 4-byte aligned, a strided 1-D
+    view, zeros, negative zeros and a NaN."""
+    g = torch.Generator().manual_seed(40 + ws)
+    lengths = [1, 2, 3, 5, 511, 1023, 1024, 1025, 2047, 2048, 2049, 4095, 4097, 6145]
+    op = ReduceOp.AVG if ws % 2 else ReduceOp.SUM
+
+    def views(bases):
+        # odd tensors start one element into their storage, every third one is strided
+        return [b[1:1 + 2 * n:2] if i % 3 == 0 else b[i % 2:i % 2 + n]
+                for i, (b, n) in enumerate(zip(bases, lengths))]
+
+    peers_cpu, peers_gpu = [], []
+    for p in range(ws):
+        bases = []
+        for n in lengths:
+            flat = torch.randn(2 * n + 3, generator=g) * (1 + p)
+            flat[::7] = 0.0
+            flat[3::11] = -0.0
+            bases.append(flat.to(dtype))
+        peers_cpu.append(views(bases))
+        peers_gpu.append(views([b.cuda() for b in bases]))
+    if dtype != torch.float32:
+        assert any(t.data_ptr() % 4 for t in peers_gpu[0])
+    assert any(t.stride(0) == 2 for t in peers_gpu[0])
+    qs_g, red_g, gath_g = sim.allreduce(q, [list(t) for t in peers_gpu], ws, op)
+    qs_c, red_c, gath_c = sim.allreduce(oracle, [list(t) for t in peers_cpu], ws, op, nthreads=NT)
+    for p, (a, b) in enumerate(zip(qs_g, qs_c)):
+        same_bytes(a, b, f"quantize peer {p}")
+    for r in red_c:
+        same_bytes(red_g[r], red_c[r], f"reduce rank {r}")
+    # dequantize into views of guard-filled storage; the storage is compared whole
+    out_c = [torch.full((2 * n + 3,), 5.0, dtype=dtype) for n in lengths]
+    out_g = [t.cuda() for t in out_c]
+    oracle.fused_dequantize_from_fp8(views(out_c), gath_c, ws, nthreads=NT)
+    q.fused_dequantize_from_fp8(views(out_g), gath_g, ws)
+    for i, (a, b) in enumerate(zip(out_g, out_c)):
+        same_bytes(a, b, f"dequantize tensor {i} (length {lengths[i]})")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("divisor", [2, 3, 7, 12, 1000, 2.5])
 def test_dequantize_with_division(q, dtype, divisor):
     """divide_by folds the caller's `tensor /= n` (manager.py:450-452) into the store of
