@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import ctypes
 import gc
+import math
 import operator
 import threading
 from collections import OrderedDict
@@ -247,8 +248,10 @@ def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor,
         else:
             # torch divides a GPU tensor by a host scalar as a multiplication by the
             # reciprocal, computed in double and rounded to fp32
+            divisor = float(divide_by)
+            factor = 1.0 / divisor if divisor != 0.0 else math.copysign(math.inf, divisor)
             _check(plan._lib.tftq_dequantize_scaled(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                                    plan.output_size, 1.0 / divide_by,
+                                                    plan.output_size, factor,
                                                     _stream_ptr(device)),
                    "tftq_dequantize_scaled")
         _keep_table(plan, device)
