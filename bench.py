@@ -101,10 +101,30 @@ def cpu_baseline(fraction: float):
                 break
     except OSError:
         pass
+    # For context: the same arithmetic written with torch CPU operators
+    # (tests/torch_restatement.py, the checker's cross-check), on 1/16 of the rows.
+    import torch_restatement as trs
+    small = workloads.cfg3(0, scale_rows=1.0 / 16)
+    small_ab = sum(workloads.algorithmic_bytes(small, ws).values())
+    small_shapes = [tuple(t.shape) if t.dim() == 2 else (t.shape[0], 1) for t in small]
+    small_outs = [torch.empty_like(t) for t in small]
+    trs_s, trs_passes = 0.0, 0
+    while trs_passes < 2 or (trs_s < 3.0 and trs_passes < 50):
+        t0 = time.perf_counter()
+        buf = trs.quantize(list(small), ws)
+        trs.reduce(small_shapes, buf.clone(), ws, 3, True)
+        trs.dequantize(small_outs, buf, ws)
+        dt = time.perf_counter() - t0
+        if trs_passes > 0:  # the first pass warms up
+            trs_s += dt
+        trs_passes += 1
+    torch_gbs = small_ab * (trs_passes - 1) / trs_s / 1e9
+
     return {
         "value": round(total / (tq + tr + td) / 1e9, 3),
         "unit": "GB/s",
         "cores": nthreads,
+        "torch_cpu_restatement_gbs": round(torch_gbs, 3),
         "kind": "port",
         "sample": f"Llama-3-8B layer bucket, {fraction:g} of the rows of each tensor at full row "
                   f"length, {passes} passes of quantize + reduce (ws=8, AVG) + dequantize, "
