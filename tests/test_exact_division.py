@@ -16,3 +16,15 @@ def test_fma_division_is_exact(tmp_path):
     res = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=600)
     assert res.returncode == 0, res.stdout
     assert " 0 mismatches" in res.stdout
+
+
+def test_three_operation_quotient_is_exact(tmp_path):
+    """Averages over a group whose size is not a power of two divide by it with a
+    multiplication and two fused multiply-adds; tests/exact_quotient.c proves by
+    exhaustion (4.3e9 quotients) that this is the correctly rounded quotient."""
+    exe = str(tmp_path / "exact_quotient")
+    subprocess.check_call(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-o", exe,
+                           os.path.join(HERE, "exact_quotient.c"), "-lm"])
+    res = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=900)
+    assert res.returncode == 0, res.stdout
+    assert " 0 mismatches" in res.stdout

@@ -285,6 +285,18 @@ def test_small_groups_several_rows_at_once(q, oracle, ws, op):
     full_check(q, oracle, peers, ws, op)
 
 
+def test_average_over_a_very_large_group(q, oracle):
+    """Group sizes from 1024 on that are not powers of two divide with the plain IEEE
+    divide (smaller ones with the three-operation quotient, powers of two with a
+    multiplication)."""
+    g = torch.Generator().manual_seed(77)
+    shapes = [(3, 300), (40,), (2, 5000)]
+    base = [[(torch.randn(s, generator=g) * (1 + p)).to(torch.bfloat16) for s in shapes] for p in range(4)]
+    for ws in (1030, 1023):
+        peers = [base[p % 4] for p in range(ws)]
+        full_check(q, oracle, peers, ws, ReduceOp.AVG, ranks=[0, ws // 2, ws - 1])
+
+
 @pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (16, ReduceOp.AVG), (24, ReduceOp.SUM),
                                    (40, ReduceOp.AVG)])
 def test_short_rows_all_team_sizes(q, oracle, ws, op):

@@ -196,8 +196,8 @@ struct KParams {
     int64_t sorted_off;
     int64_t map_off;
     Dealt dealt;        // inline table only
-    int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG general
+    int32_t div_mode;   // reduce: 0 = SUM, 1 = AVG with power-of-two ws, 2 = AVG, other ws < 1024, 3 = AVG, larger ws
     float div;          // reduce: 1.0 or float(ws)
-    float inv_div;      // reduce: exact reciprocal when div_mode == 1
+    float inv_div;      // reduce: RN(1 / div); exact when div_mode == 1
     float post_scale;   // dequantize: factor applied to the rounded result (scaled variant only)
 };

@@ -58,14 +58,26 @@ DEV void accumulate16(float (&acc)[16], const u32x4 w, float r, float r_lo)
     }
 }
 
-// (acc * s2) / div, left to right (:364).  GDIV: div is not a power of two
-// and needs a real divide; otherwise inv_div (1 for SUM) is an exact inverse
-// and multiplying by it is the same correctly rounded result.
-template <bool GDIV>
+// (acc * s2) / div, left to right (:364).  Without GDIV, inv_div (1 for SUM) is
+// the exact inverse of a power of two and multiplying by it is the same
+// correctly rounded result.  GDIV: div is not a power of two.  For div < 1024
+// the quotient comes from inv_div = RN(1 / div) in three operations,
+//     q0 = y * inv_div,  rem = fma(-q0, div, y),  q = fma(rem, inv_div, q0),
+// which equals RN(y / div) for every binary32 y whose quotient is not close to
+// the subnormal range (tests/exact_quotient.c checks all 2^23 mantissas of y
+// against every odd div below 1024; powers of two in div only move exponents).
+// Below 2^-100 the steps may round differently, but every |q| < 2^-10 gives the
+// code +-0, with the sign of y restored by the copysign (-0 / div = -0).
+// IEEE: the plain divide, for larger group sizes (div_mode 3).
+template <bool GDIV, bool IEEE = false>
 DEV float scale_div(float a, float s2, const KParams &p)
 {
     const float y = a * s2;
-    return GDIV ? y / p.div : y * p.inv_div;
+    if (!GDIV) return y * p.inv_div;
+    if (IEEE) return y / p.div;
+    const float q0 = y * p.inv_div;
+    const float rem = __builtin_fmaf(-q0, p.div, y);
+    return __builtin_copysignf(__builtin_fmaf(rem, p.inv_div, q0), y);
 }
 
 // row maximum / div (:340); for a power-of-two div the multiplication by the
@@ -117,7 +129,7 @@ DEV float guarded_scale(GLOBAL const u32 *prow)
 // One column at a time with plain IEEE divides, two passes: the path of rows
 // in which some peer's scale is outside the range of the fast exact division,
 // and of rows too long for registers.  Small code, not tuned.
-template <int TEAM, bool GDIV>
+template <int TEAM, bool GDIV, bool IEEE = false>
 DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float *lds)
 {
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
@@ -138,7 +150,7 @@ DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float 
             if (pass == 0) {
                 amax = fmaxf(amax, __builtin_fabsf(a));
             } else {
-                const float y = scale_div<GDIV>(a, s2, p);
+                const float y = scale_div<GDIV, IEEE>(a, s2, p);
                 orow[4 + c] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(y, 0.0f, 0, false) & 0xFF);
             }
         }
@@ -562,7 +574,7 @@ DEV void reduce_rows_at_once(const Seg &s, const KParams &p, int j0, int lane, f
 
 // Rows of one column: 8 bytes per row and peer, one plain divide per peer
 // (coefficients for the fast division would cost two), four rows per lane.
-template <bool GDIV>
+template <bool GDIV, bool IEEE = false>
 DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 {
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -588,7 +600,7 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
             const float s2 = calc_scale(amax_div<GDIV>(fmaxf(0.0f, __builtin_fabsf(acc[k])), p));  // NaN ignored (:331-338)
             u32x2 o;
             o.x = as_u(s2);
-            o.y = pack_fp8x4(scale_div<GDIV>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
+            o.y = pack_fp8x4(scale_div<GDIV, IEEE>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
             *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off[k]) = o;
         }
     }
@@ -604,6 +616,31 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
     const int blk = vb - s.wg_begin[ST_R];
     const int tid = threadIdx.x;
     const int ndw = (s.row_bytes >> 2) - 1;
+    if (GDIV && p.div_mode == 3) {
+        // averages over 1024 peers or more, not a power of two: the untuned path with plain divides
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        switch (s.kind[ST_R]) {
+        case K_GEN256: reduce_row_slow<256, true, true>(s, p, blk, tid, lds); break;
+        case K_GEN64:
+            if (blk * 4 + wave < s.slice_rows) reduce_row_slow<64, true, true>(s, p, blk * 4 + wave, tid & 63, lds);
+            break;
+        case K_GEN32:
+            if (blk * 8 + (tid >> 5) < s.slice_rows) reduce_row_slow<32, true, true>(s, p, blk * 8 + (tid >> 5), tid & 31, lds);
+            break;
+        case K_GEN16:
+            if (blk * 16 + (tid >> 4) < s.slice_rows) reduce_row_slow<16, true, true>(s, p, blk * 16 + (tid >> 4), tid & 15, lds);
+            break;
+        case K_GEN8:
+            if (blk * 32 + (tid >> 3) < s.slice_rows) reduce_row_slow<8, true, true>(s, p, blk * 32 + (tid >> 3), tid & 7, lds);
+            break;
+        case K_GEN1:
+            if (blk * 256 + tid < s.slice_rows) reduce_row_slow<1, true, true>(s, p, blk * 256 + tid, 0, lds);
+            break;
+        case K_COL1: reduce_col1<true, true>(s, p, blk * tftq_col1_rows_per_wg(ST_R), tid); break;
+        default: break;
+        }
+        return;
+    }
     switch (s.kind[ST_R]) {
     case K_GEN256: {  // one workgroup per row, or per 2 or 4 rows when the group is small
         const int rows = tftq_reduce_rows_at_once(K_GEN256, ndw, p.ws);
@@ -710,14 +747,17 @@ extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_b
         if ((ws & (ws - 1)) == 0) {
             kp.div_mode = 1;
             kp.inv_div = 1.0f / (float)ws;
-        } else {
+        } else if (ws < 1024) {
             kp.div_mode = 2;
+            kp.inv_div = 1.0f / (float)ws;
+        } else {
+            kp.div_mode = 3;
         }
     }
     if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid(grid_of(kp)), block(TFTQ_WG);
-    const bool gdiv = kp.div_mode == 2;
+    const bool gdiv = kp.div_mode >= 2;
 #define TFTQ_LAUNCH_R(I, G, W) hipLaunchKernelGGL((k_reduce<I, G, W>), grid, block, 0, st, kp, inl)
     if (plan->wide[ST_R]) {
         if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, true); else TFTQ_LAUNCH_R(false, true, true); }
