@@ -368,6 +368,27 @@ def test_wide_rows(q, oracle):
         full_check(q, oracle, peers[:3], 3, ReduceOp.AVG, ranks=[2])
 
 
+def test_rows_parked_in_lds(q, oracle):
+    """Rows of 4097 to 7936 input vectors (16-bit: 32776 to 63488 columns, fp32: 16388 to
+    31744): the quantize kernel keeps 16 vectors per lane in registers and parks the rest in
+    LDS.  Both ends of the range, the first length beyond it (two passes), a tail after the
+    last whole vector, a row that does not start on a 16-byte boundary, padding rows."""
+    g = torch.Generator().manual_seed(29)
+    for dtype, cols in ((torch.bfloat16, [32776, 40001, 53248, 63488, 63493, 63496]),
+                        (torch.float16, [53248, 63489]),
+                        (torch.float32, [16388, 28672, 31744, 31747, 31748])):
+        peers = []
+        for p in range(2):
+            ts = [torch.randn(3, c, generator=g).to(dtype) * (p + 1) for c in cols]
+            flat = torch.randn(2 * 40001 + 1, generator=g).to(dtype)
+            ts.append(flat[1:].view(2, 40001))
+            ts.append(torch.randn(70, 512, generator=g).to(dtype))
+            peers.append(ts)
+        peers[1][0][1] *= 1e-30
+        peers[0][1][2] = 0.0
+        full_check(q, oracle, peers, 2, ReduceOp.AVG)
+
+
 def test_long_rows(q, oracle):
     """Rows longer than the register-resident paths hold: 20000 and 70000 columns."""
     g = torch.Generator().manual_seed(21)

@@ -106,9 +106,13 @@ constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel argumen
 // Rows a workgroup can hold in registers.  The regular kernels keep up to 8
 // input vectors per lane in quantize (rows of 2048 vectors = 32 KB) and the
 // accumulators of 4096 payload dwords (16384 columns) in reduce; the "wide"
-// kernel variants hold twice that at half the occupancy and are launched only
-// for plans that contain such rows.  Longer rows make two passes.
+// kernel variants hold twice that at half the occupancy, the wide quantize kernel
+// parks another 15 vectors per lane in LDS (rows of up to 7936 vectors = 124 KB:
+// 63488 bf16 or 31744 fp32 columns), and they are launched only for plans that
+// contain such rows.  Longer rows make two passes.
 constexpr int TFTQ_Q_VECS = 8 * TFTQ_WG, TFTQ_Q_VECS_WIDE = 16 * TFTQ_WG;
+constexpr int TFTQ_Q_PARKED = 15;  // more vectors per lane that the wide quantize kernel parks in LDS (60 KB)
+constexpr int TFTQ_Q_VECS_LDS = TFTQ_Q_VECS_WIDE + TFTQ_Q_PARKED * TFTQ_WG;
 constexpr int TFTQ_R_DWORDS = 4096, TFTQ_R_DWORDS_WIDE = 8192;
 
 // One tensor of the list.  64 bytes.
@@ -173,6 +177,7 @@ struct tftq_plan {
     int64_t max_rows;
     int32_t nwg[3];
     bool wide[3];              // per stage: some row needs the kernel variant with more registers
+    bool parked;               // quantize: some row also needs the 60 KB of LDS (rows above TFTQ_Q_VECS_WIDE)
     Dealt dealt[3];            // inline table only
     int32_t dealt_per_xcd[3];  // inline table only: workgroups of the busiest XCD
     TableIndex index[3];       // device table only

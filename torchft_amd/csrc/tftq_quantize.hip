@@ -149,14 +149,98 @@ DEV void quantize_vec_long(const Seg &s, const KParams &p, int row, int tid, flo
     }
 }
 
+// Rows of 4097 to 7936 vectors (64 to 124 KB; wide kernel only): the first 16
+// vectors of a lane stay in registers, up to 15 more are parked in LDS, where
+// every lane reads back only what it wrote itself, so the row is still read
+// from memory once.  The parked vectors travel in three groups of five; the
+// loads of the next group are issued before the current one is parked.
+template <typename T>
+DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, float *lds, u32x4 *park)
+{
+    constexpr int KR = 2 * QV, G = 5, NG = TFTQ_Q_PARKED / G;
+    static_assert(NG * G == TFTQ_Q_PARKED, "groups of five");
+    const bool active = row < s.slice_rows * p.ws;
+    GLOBAL u32 *out = as_global<u32>(p.packed + (active ? row_addr(s, p.slot_size, row) : 0));
+    if (active && row >= s.m) {
+        for (int d = tid; d < (s.row_bytes >> 2); d += TFTQ_WG) out[d] = 0;  // padding row
+    }
+    if (!active || row >= s.m) return;  // the whole workgroup leaves
+
+    constexpr int EPV = Elem<T>::EPV;
+    const int nvec = s.n / EPV;
+    const int tail = s.n - nvec * EPV;
+    const int64_t r0 = (int64_t)row * s.row_stride;
+    GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
+    u32x4 v[KR], w[2][G];
+#pragma unroll
+    for (int k = 0; k < KR; k++) v[k] = LOAD_STREAM(in + min(k * TFTQ_WG + tid, nvec - 1));
+#pragma unroll
+    for (int k = 0; k < G; k++) w[0][k] = LOAD_STREAM(in + min((KR + k) * TFTQ_WG + tid, nvec - 1));
+    float t[EPV - 1];
+    if (tail) {
+#pragma unroll
+        for (int e = 0; e < EPV - 1; e++) t[e] = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(e, tail - 1));
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KR; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        if (g + 1 < NG) {
+#pragma unroll
+            for (int k = 0; k < G; k++)
+                w[(g + 1) & 1][k] = LOAD_STREAM(in + min((KR + (g + 1) * G + k) * TFTQ_WG + tid, nvec - 1));
+        }
+#pragma unroll
+        for (int k = 0; k < G; k++) {
+            amax = fmaxf(amax, vec_absmax<T>(w[g & 1][k]));
+            park[(g * G + k) * TFTQ_WG + tid] = w[g & 1][k];
+        }
+    }
+    if (tail) {
+#pragma unroll
+        for (int e = 0; e < EPV - 1; e++) amax = fmaxf(amax, __builtin_fabsf(t[e]));
+    }
+    amax = team_max<256>(amax, lds);
+    const float sc = calc_scale(amax);
+    if (tid == 0) out[0] = as_u(sc);
+#pragma unroll
+    for (int k = 0; k < KR; k++) asm volatile("" : "+v"(v[k].x), "+v"(v[k].y), "+v"(v[k].z), "+v"(v[k].w));
+#pragma unroll
+    for (int k = 0; k < KR; k++) {
+        const int idx = k * TFTQ_WG + tid;
+        if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
+    }
+#pragma unroll
+    for (int k = 0; k < TFTQ_Q_PARKED; k++) {
+        const int idx = (KR + k) * TFTQ_WG + tid;
+        if (idx < nvec) vec_quant_store<T>(park[k * TFTQ_WG + tid], sc, out + 1, idx);
+    }
+    if (tail && tid == 0) {
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) y[e] = (e < EPV - 1 && e < tail) ? t[e < EPV - 1 ? e : 0] * sc : 0.0f;
+        GLOBAL u32 *tw = out + 1 + nvec * (EPV / 4);
+        u32 w0 = pack_fp8x4(y[0], y[1], y[2], y[3]);
+        if (tail < 4) w0 &= (1u << (8 * tail)) - 1u;
+        tw[0] = w0;
+        if (EPV == 8 && tail > 4) {
+            u32 w1 = pack_fp8x4(y[4], y[5], y[6], y[7]);
+            if (tail < 8) w1 &= (1u << (8 * (tail - 4))) - 1u;
+            tw[1] = w1;
+        }
+    }
+}
+
 template <typename T, int TEAM, bool WIDE>
-DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds)
+DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *lds, u32x4 *park)
 {
     // same branch for the whole workgroup
     const int nvec = s.n / Elem<T>::EPV;
     if (nvec <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
     else if (TEAM < 256 || nvec <= TFTQ_Q_VECS) quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
     else if (WIDE && nvec <= TFTQ_Q_VECS_WIDE) quantize_vec_k<T, TEAM, 2 * QV>(s, p, row, lane, lds);
+    else if (WIDE && nvec <= TFTQ_Q_VECS_LDS) quantize_vec_lds<T>(s, p, row, lane, lds, park);
     else quantize_vec_long<T>(s, p, row, lane, lds);
 }
 
@@ -338,19 +422,22 @@ template <typename T, bool INLINE, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
+    // 60 KB of dynamic LDS, asked for at the launch only when the plan has rows that need it
+    // (it limits a CU to two workgroups)
+    extern __shared__ u32x4 park[];
     Seg s;
     int vb;
     if (!locate<INLINE, ST_Q>(p, inl, s, vb)) return;
     const int blk = vb - s.wg_begin[ST_Q];
     const int tid = threadIdx.x;
     switch (s.kind[ST_Q]) {
-    case K_VEC256: quantize_vec<T, 256, WIDE>(s, p, blk, tid, lds); break;
+    case K_VEC256: quantize_vec<T, 256, WIDE>(s, p, blk, tid, lds, park); break;
     case K_VEC64:
-        quantize_vec<T, 64, false>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds);
+        quantize_vec<T, 64, false>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds, park);
         break;
-    case K_VEC32: quantize_vec<T, 32, false>(s, p, blk * 8 + (tid >> 5), tid & 31, lds); break;
-    case K_VEC16: quantize_vec<T, 16, false>(s, p, blk * 16 + (tid >> 4), tid & 15, lds); break;
-    case K_VEC8: quantize_vec<T, 8, false>(s, p, blk * 32 + (tid >> 3), tid & 7, lds); break;
+    case K_VEC32: quantize_vec<T, 32, false>(s, p, blk * 8 + (tid >> 5), tid & 31, lds, park); break;
+    case K_VEC16: quantize_vec<T, 16, false>(s, p, blk * 16 + (tid >> 4), tid & 15, lds, park); break;
+    case K_VEC8: quantize_vec<T, 8, false>(s, p, blk * 32 + (tid >> 3), tid & 7, lds, park); break;
     case K_GEN64:
         quantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;
@@ -363,12 +450,14 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
 }
 
 template <typename T>
-static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, hipStream_t st)
+static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, bool parked,
+                    hipStream_t st)
 {
     const dim3 grid(grid_of(kp)), block(TFTQ_WG);
     if (wide) {
-        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, true>), grid, block, 0, st, kp, inl);
-        else hipLaunchKernelGGL((k_quantize<T, false, true>), grid, block, 0, st, kp, inl);
+        const unsigned lds = parked ? TFTQ_Q_PARKED * TFTQ_WG * 16u : 0u;
+        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, true>), grid, block, lds, st, kp, inl);
+        else hipLaunchKernelGGL((k_quantize<T, false, true>), grid, block, lds, st, kp, inl);
     } else {
         if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, false>), grid, block, 0, st, kp, inl);
         else hipLaunchKernelGGL((k_quantize<T, false, false>), grid, block, 0, st, kp, inl);
@@ -389,9 +478,9 @@ extern "C" int tftq_quantize(const tftq_plan *plan, void *packed, int64_t packed
     if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
     switch (plan->dtype) {
-    case TFTQ_F32: return launch_q<float>(kp, inl, use_inline, plan->wide[ST_Q], st);
-    case TFTQ_F16: return launch_q<f16_tag>(kp, inl, use_inline, plan->wide[ST_Q], st);
-    case TFTQ_BF16: return launch_q<bf16_tag>(kp, inl, use_inline, plan->wide[ST_Q], st);
+    case TFTQ_F32: return launch_q<float>(kp, inl, use_inline, plan->wide[ST_Q], plan->parked, st);
+    case TFTQ_F16: return launch_q<f16_tag>(kp, inl, use_inline, plan->wide[ST_Q], plan->parked, st);
+    case TFTQ_BF16: return launch_q<bf16_tag>(kp, inl, use_inline, plan->wide[ST_Q], plan->parked, st);
     default: return TFTQ_E_DTYPE;
     }
 }
