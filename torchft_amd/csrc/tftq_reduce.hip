@@ -168,26 +168,26 @@ DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float 
 // Rows longer than a 256-lane team can keep in registers (more than 16384
 // columns): two passes over chunks of 1024 dwords, as the reference does for
 // every row (:318-372), but with 16-byte loads, the fast exact division and the
-// scales read once.  The second pass finds the peer rows in the caches.
-template <bool GDIV>
-DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *lds)
+// scales read once.  The second pass reads the peer rows again (from the
+// caches if they are still there).
+// The passes cover the dwords from d0 on; the caller has dealt with the dwords
+// before d0, hands in their maximum and stores them in `between`, which runs
+// when the new scale is known and every lane has finished reading for the
+// first pass.  c: division coefficients of peer min(lane, ws - 1), all fast.
+template <bool GDIV, typename Between>
+DEV void reduce_row_two_passes(const Seg &s, const KParams &p, int j, int tid, float *lds, const DivCoef &c,
+                               int d0, float amax, Between between)
 {
     const int ndw = (s.row_bytes >> 2) - 1;
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
-    const int wlane = tid & 63;
     const int ws = p.ws;  // <= 64 here
-    const DivCoef c = make_div(guarded_scale(peer_row(p, min(wlane, ws - 1), off)));
-    if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // same in the four wavefronts
-        reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
-        return;
-    }
     GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
     const u32 tailmask = (s.n & 3) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
-    float amax = 0.0f, s2 = 0.0f;
+    float s2 = 0.0f;
 #pragma nounroll
     for (int pass = 0; pass < 2; pass++) {
 #pragma nounroll
-        for (int d = 0; d < ndw; d += 4 * TFTQ_WG) {
+        for (int d = d0; d < ndw; d += 4 * TFTQ_WG) {
             const bool valid = d + 4 * tid < ndw;
             const int doff = min(d + 4 * tid, ndw - 4);  // the last vector ends with the row
             const u32 mask = doff == ndw - 4 ? tailmask : 0xFFFFFFFFu;
@@ -219,9 +219,9 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
                     if (doff >= d) {
                         *(GLOBAL u32x4_a4 *)(orow + 1 + doff) = o;
                     } else {
-                        // The vector reaches back into the previous chunk, whose codes have
-                        // already been replaced in the own slot: what was accumulated for
-                        // those dwords is meaningless and they are final already.
+                        // The vector reaches back into the dwords before this chunk, whose
+                        // codes have already been replaced in the own slot: what was
+                        // accumulated for those dwords is meaningless and they are final already.
 #pragma unroll
                         for (int e = 0; e < 4; e++)
                             if (doff + e >= d) orow[1 + doff + e] = o[e];
@@ -232,9 +232,65 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
         if (pass == 0) {
             amax = team_max<256>(amax, lds);  // every wavefront has read the old scales by now
             s2 = calc_scale(amax_div<GDIV>(amax, p));
+            between(s2);
         }
     }
     if (tid == 0) orow[0] = as_u(s2);  // :375
+}
+
+template <bool GDIV>
+DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *lds)
+{
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    const DivCoef c = make_div(guarded_scale(peer_row(p, min(tid & 63, p.ws - 1), off)));
+    if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // same in the four wavefronts
+        reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
+        return;
+    }
+    reduce_row_two_passes<GDIV>(s, p, j, tid, lds, c, 0, 0.0f, [](float) {});
+}
+
+// Wide kernel, rows of more than 8192 payload dwords: the sums of the first 8192
+// dwords stay in registers (128 per lane) and only the rest of the row makes two
+// passes, so the peers are read 1 + rest / length times instead of twice
+// (53248 columns: 1.38 times).
+template <bool GDIV>
+DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float *lds)
+{
+    constexpr int UNITS = TFTQ_R_DWORDS_WIDE / (4 * TFTQ_WG);  // 8
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    const int ws = p.ws;  // <= 64 here
+    const DivCoef c = make_div(guarded_scale(peer_row(p, min(tid & 63, ws - 1), off)));
+    if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // same in the four wavefronts
+        reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
+        return;
+    }
+    float acc[UNITS][16];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+#pragma nounroll
+    for (int k = 0; k < ws; k++) {
+        GLOBAL const u32 *pv = peer_row(p, k, off) + 1;
+        u32x4 w[UNITS];
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + 4 * (u * TFTQ_WG + tid)));
+        const float pr = bcast_lane(c.r, k), pl = bcast_lane(c.r_lo, k);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) accumulate16(acc[u], w[u], pr, pl);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+    GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+    reduce_row_two_passes<GDIV>(s, p, j, tid, lds, c, TFTQ_R_DWORDS_WIDE, amax, [&](float s2) {
+#pragma unroll
+        for (int u = 0; u < UNITS; u++)
+            *(GLOBAL u32x4_a4 *)(orow + 1 + 4 * (u * TFTQ_WG + tid)) = requant16<GDIV>(acc[u], s2, p);
+    });
 }
 
 // Register-resident row: the team holds all accumulators of the row, each peer
@@ -654,6 +710,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
             reduce_rows<256, 8, false, GDIV>(s, p, j, tid, lds);
         } else if (ndw > TFTQ_R_DWORDS) {
             if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
+            else if (WIDE && ndw > TFTQ_R_DWORDS_WIDE) reduce_row_hybrid<GDIV>(s, p, j, tid, lds);
             else reduce_row_long<GDIV>(s, p, j, tid, lds);
         } else if (p.ws > 64) {
             if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j, tid, lds);
