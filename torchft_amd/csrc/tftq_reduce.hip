@@ -174,9 +174,11 @@ DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float 
 // before d0, hands in their maximum and stores them in `between`, which runs
 // when the new scale is known and every lane has finished reading for the
 // first pass.  c: division coefficients of peer min(lane, ws - 1), all fast.
-template <bool GDIV, typename Between>
+// PARK: the sums of the first PARK chunks are parked in LDS (parked: PARK * 16 KB) by the
+// first pass and taken from there by the second, which then reads no peer for them.
+template <bool GDIV, int PARK, typename Between>
 DEV void reduce_row_two_passes(const Seg &s, const KParams &p, int j, int tid, float *lds, const DivCoef &c,
-                               int d0, float amax, Between between)
+                               int d0, float amax, Between between, float *parked = nullptr)
 {
     const int ndw = (s.row_bytes >> 2) - 1;
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
@@ -191,25 +193,36 @@ DEV void reduce_row_two_passes(const Seg &s, const KParams &p, int j, int tid, f
             const bool valid = d + 4 * tid < ndw;
             const int doff = min(d + 4 * tid, ndw - 4);  // the last vector ends with the row
             const u32 mask = doff == ndw - 4 ? tailmask : 0xFFFFFFFFu;
+            const int chunk = (d - d0) / (4 * TFTQ_WG);
+            const bool in_lds = PARK > 0 && chunk < PARK;  // same for the whole workgroup
             float acc[16];
+            if (pass == 1 && in_lds) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+                for (int e = 0; e < 16; e++) acc[e] = parked[(chunk * 16 + e) * TFTQ_WG + tid];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[e] = 0.0f;
 #pragma nounroll
-            for (int k0 = 0; k0 < ws; k0 += 4) {
-                u32x4 w[4];
+                for (int k0 = 0; k0 < ws; k0 += 4) {
+                    u32x4 w[4];
 #pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k0 + b, ws - 1), off) + 1 + doff));
-                }
+                    for (int b = 0; b < 4; b++) {
+                        w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k0 + b, ws - 1), off) + 1 + doff));
+                    }
 #pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    w[b].w &= mask;
-                    if (k0 + b < ws) accumulate16(acc, w[b], bcast_lane(c.r, k0 + b), bcast_lane(c.r_lo, k0 + b));
+                    for (int b = 0; b < 4; b++) {
+                        w[b].w &= mask;
+                        if (k0 + b < ws) accumulate16(acc, w[b], bcast_lane(c.r, k0 + b), bcast_lane(c.r_lo, k0 + b));
+                    }
                 }
             }
             if (pass == 0) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[e]));
+                if (in_lds) {  // every lane reads back only what it wrote
+#pragma unroll
+                    for (int e = 0; e < 16; e++) parked[(chunk * 16 + e) * TFTQ_WG + tid] = acc[e];
+                }
             } else {
                 // the moved-back last vector overlaps its neighbour, which may sit in another
                 // wavefront: nobody stores before everybody has read the own slot's chunk
@@ -247,15 +260,16 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
         reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
         return;
     }
-    reduce_row_two_passes<GDIV>(s, p, j, tid, lds, c, 0, 0.0f, [](float) {});
+    reduce_row_two_passes<GDIV, 0>(s, p, j, tid, lds, c, 0, 0.0f, [](float) {});
 }
 
 // Wide kernel, rows of more than 8192 payload dwords: the sums of the first 8192
-// dwords stay in registers (128 per lane) and only the rest of the row makes two
-// passes, so the peers are read 1 + rest / length times instead of twice
-// (53248 columns: 1.38 times).
+// dwords stay in registers (128 per lane), those of the next 3072 are parked in
+// 48 KB of LDS and only the rest of the row makes two passes, so the peers are
+// read 1 + rest / length times instead of twice (53248 columns: 1.15 times).
+constexpr int R_PARKED_CHUNKS = 3;  // chunks of 1024 dwords = 16 KB of sums each
 template <bool GDIV>
-DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float *lds)
+DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float *lds, float *parked)
 {
     constexpr int UNITS = TFTQ_R_DWORDS_WIDE / (4 * TFTQ_WG);  // 8
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
@@ -286,11 +300,11 @@ DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float
 #pragma unroll
         for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
     GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
-    reduce_row_two_passes<GDIV>(s, p, j, tid, lds, c, TFTQ_R_DWORDS_WIDE, amax, [&](float s2) {
+    reduce_row_two_passes<GDIV, R_PARKED_CHUNKS>(s, p, j, tid, lds, c, TFTQ_R_DWORDS_WIDE, amax, [&](float s2) {
 #pragma unroll
         for (int u = 0; u < UNITS; u++)
             *(GLOBAL u32x4_a4 *)(orow + 1 + 4 * (u * TFTQ_WG + tid)) = requant16<GDIV>(acc[u], s2, p);
-    });
+    }, parked);
 }
 
 // Register-resident row: the team holds all accumulators of the row, each peer
@@ -666,6 +680,7 @@ template <bool INLINE, bool GDIV, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[16];
+    __shared__ float parked[WIDE ? R_PARKED_CHUNKS * 16 * TFTQ_WG : 1];  // wide kernel: 48 KB (two workgroups per CU fit)
     Seg s;
     int vb;
     if (!locate<INLINE, ST_R>(p, inl, s, vb)) return;
@@ -710,7 +725,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
             reduce_rows<256, 8, false, GDIV>(s, p, j, tid, lds);
         } else if (ndw > TFTQ_R_DWORDS) {
             if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
-            else if (WIDE && ndw > TFTQ_R_DWORDS_WIDE) reduce_row_hybrid<GDIV>(s, p, j, tid, lds);
+            else if (WIDE && ndw > TFTQ_R_DWORDS_WIDE) reduce_row_hybrid<GDIV>(s, p, j, tid, lds, parked);
             else reduce_row_long<GDIV>(s, p, j, tid, lds);
         } else if (p.ws > 64) {
             if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j, tid, lds);
