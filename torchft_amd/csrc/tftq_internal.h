@@ -109,7 +109,7 @@ constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel argumen
 // kernel variants hold twice that at half the occupancy, the wide quantize kernel
 // parks another 15 vectors per lane in LDS (rows of up to 7936 vectors = 124 KB:
 // 63488 bf16 or 31744 fp32 columns), and they are launched only for plans that
-// contain such rows.  Longer rows make two passes.
+// contain such rows.  What a row has beyond that is read twice.
 constexpr int TFTQ_Q_VECS = 8 * TFTQ_WG, TFTQ_Q_VECS_WIDE = 16 * TFTQ_WG;
 constexpr int TFTQ_Q_PARKED = 15;  // more vectors per lane that the wide quantize kernel parks in LDS (60 KB)
 constexpr int TFTQ_Q_VECS_LDS = TFTQ_Q_VECS_WIDE + TFTQ_Q_PARKED * TFTQ_WG;

@@ -295,8 +295,8 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
     for (int i = 0; i < n_tensors; i++) {
         const Seg &s = p->segs[(size_t)i];
         const int nvec = s.n / (16 / p->esz), ndw = s.row_bytes / 4 - 1;
-        if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS && nvec <= TFTQ_Q_VECS_LDS && s.m > 0) p->wide[ST_Q] = true;
-        if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS_WIDE && nvec <= TFTQ_Q_VECS_LDS && s.m > 0) p->parked = true;
+        if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS && s.m > 0) p->wide[ST_Q] = true;
+        if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS_WIDE && s.m > 0) p->parked = true;
         if (s.kind[ST_R] == K_GEN256 && ndw > TFTQ_R_DWORDS && s.m > 0 && ws <= 64)
             p->wide[ST_R] = true;
     }

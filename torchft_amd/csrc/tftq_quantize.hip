@@ -98,62 +98,13 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     }
 }
 
-// Rows of more than 32 KB: too long for the registers of a workgroup.  Two
-// passes with 16-byte loads; the second one finds the row in the caches.
-template <typename T>
-DEV void quantize_vec_long(const Seg &s, const KParams &p, int row, int tid, float *lds)
-{
-    const bool active = row < s.slice_rows * p.ws;
-    if (!active) return;
-    GLOBAL u32 *out = as_global<u32>(p.packed + row_addr(s, p.slot_size, row));
-    if (row >= s.m) {
-        for (int d = tid; d < (s.row_bytes >> 2); d += TFTQ_WG) out[d] = 0;
-        return;
-    }
-    constexpr int EPV = Elem<T>::EPV;
-    const int nvec = s.n / EPV;
-    const int64_t r0 = (int64_t)row * s.row_stride;
-    GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
-    float amax = 0.0f;
-    for (int c = nvec * EPV + tid; c < s.n; c += TFTQ_WG) amax = fmaxf(amax, __builtin_fabsf(Elem<T>::load(s.ptr, r0 + c)));
-#pragma nounroll
-    for (int base = 0; base < nvec; base += 4 * TFTQ_WG) {
-        u32x4 v[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) v[k] = in[min(base + k * TFTQ_WG + tid, nvec - 1)];
-#pragma unroll
-        for (int k = 0; k < 4; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
-    }
-    amax = team_max<256>(amax, lds);
-    const float sc = calc_scale(amax);
-    if (tid == 0) out[0] = as_u(sc);
-#pragma nounroll
-    for (int base = 0; base < nvec; base += 4 * TFTQ_WG) {
-        u32x4 v[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) v[k] = LOAD_STREAM(in + min(base + k * TFTQ_WG + tid, nvec - 1));
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int idx = base + k * TFTQ_WG + tid;
-            if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
-        }
-    }
-    // tail: at most EPV - 1 elements after the last whole vector, byte stores plus zero padding
-    if (tid == 0) {
-        const int c0 = nvec * EPV;
-        GLOBAL uint8_t *ob = (GLOBAL uint8_t *)(out + 1);
-        for (int c = c0; c < ((s.n + 3) & ~3); c++) {
-            const float x = c < s.n ? Elem<T>::load(s.ptr, r0 + c) : 0.0f;
-            ob[c] = c < s.n ? (uint8_t)(pack_fp8x4(x * sc, 0.0f, 0.0f, 0.0f) & 0xFFu) : (uint8_t)0;
-        }
-    }
-}
-
-// Rows of 4097 to 7936 vectors (64 to 124 KB; wide kernel only): the first 16
+// Rows of more than 4096 vectors (64 KB; wide kernel only): the first 16
 // vectors of a lane stay in registers, up to 15 more are parked in LDS, where
-// every lane reads back only what it wrote itself, so the row is still read
-// from memory once.  The parked vectors travel in three groups of five; the
-// loads of the next group are issued before the current one is parked.
+// every lane reads back only what it wrote itself, so rows of up to 7936
+// vectors (124 KB) are still read from memory once.  The parked vectors travel
+// in three groups of five; the loads of the next group are issued before the
+// current one is parked.  What a longer row has beyond 7936 vectors is read
+// twice, once for the maximum and once to be quantized.
 template <typename T>
 DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, float *lds, u32x4 *park)
 {
@@ -201,6 +152,14 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
 #pragma unroll
         for (int e = 0; e < EPV - 1; e++) amax = fmaxf(amax, __builtin_fabsf(t[e]));
     }
+#pragma nounroll
+    for (int base = TFTQ_Q_VECS_LDS; base < nvec; base += 4 * TFTQ_WG) {  // first pass over the rest
+        u32x4 x[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) x[k] = in[min(base + k * TFTQ_WG + tid, nvec - 1)];
+#pragma unroll
+        for (int k = 0; k < 4; k++) amax = fmaxf(amax, vec_absmax<T>(x[k]));
+    }
     amax = team_max<256>(amax, lds);
     const float sc = calc_scale(amax);
     if (tid == 0) out[0] = as_u(sc);
@@ -215,6 +174,17 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
     for (int k = 0; k < TFTQ_Q_PARKED; k++) {
         const int idx = (KR + k) * TFTQ_WG + tid;
         if (idx < nvec) vec_quant_store<T>(park[k * TFTQ_WG + tid], sc, out + 1, idx);
+    }
+#pragma nounroll
+    for (int base = TFTQ_Q_VECS_LDS; base < nvec; base += 4 * TFTQ_WG) {  // second pass over the rest
+        u32x4 x[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) x[k] = LOAD_STREAM(in + min(base + k * TFTQ_WG + tid, nvec - 1));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int idx = base + k * TFTQ_WG + tid;
+            if (idx < nvec) vec_quant_store<T>(x[k], sc, out + 1, idx);
+        }
     }
     if (tail && tid == 0) {
         float y[8];
@@ -240,8 +210,8 @@ DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *
     if (nvec <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2>(s, p, row, lane, lds);
     else if (TEAM < 256 || nvec <= TFTQ_Q_VECS) quantize_vec_k<T, TEAM, QV>(s, p, row, lane, lds);
     else if (WIDE && nvec <= TFTQ_Q_VECS_WIDE) quantize_vec_k<T, TEAM, 2 * QV>(s, p, row, lane, lds);
-    else if (WIDE && nvec <= TFTQ_Q_VECS_LDS) quantize_vec_lds<T>(s, p, row, lane, lds, park);
-    else quantize_vec_long<T>(s, p, row, lane, lds);
+    else if (WIDE) quantize_vec_lds<T>(s, p, row, lane, lds, park);
+    // else: the planner launches the wide kernel, with its LDS, for plans that have such rows
 }
 
 // Any strides, any alignment, any n: element loads, two passes over the row
