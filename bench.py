@@ -33,7 +33,6 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 
@@ -45,10 +44,12 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--sets", type=int, default=3, help="buffer sets the steps rotate over")
     ap.add_argument("--rank", type=int, default=None)
-    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat", "shape"],
+    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat", "shape", "ceiling"],
                     help="workload: 3 = Llama-3-8B layer bucket (the headline, default); 2, 4, 5 = the "
                          "other GPU configurations; flat = one 1-D fp32 tensor of 64 Mi elements "
-                         "(what a bucketised DiLoCo all-reduce passes); shape = --shape")
+                         "(what a bucketised DiLoCo all-reduce passes); shape = --shape; ceiling = "
+                         "streaming kernels without arithmetic for the read : write mixes of the "
+                         "stages, at the headline workload's footprint, beside the product kernels")
     ap.add_argument("--shape", default="53248x4096",
                     help="with --config shape: ROWSxCOLS[,ROWSxCOLS...], N(0, 0.02) values")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16", "float32"],
@@ -136,12 +137,140 @@ def cpu_baseline(fraction: float):
     }
 
 
+def run_ceilings(args) -> int:
+    """Streaming ceilings (torchft_amd/csrc/tftq_ceiling.hip) at the footprint of the headline
+    workload, and the three product kernels timed the same way: every kernel alone in a loop
+    that rotates over `--sets` buffer sets (cold last-level cache), HIP events around each
+    launch on the launch stream."""
+    import ctypes
+
+    import torch
+    from torch.distributed import ReduceOp
+
+    import workloads
+    from torchft_amd import _build, _lib, quantization as q
+
+    torch.cuda.set_device(0)
+    dev = "cuda"
+    if not os.path.exists(_build.CEILING_LIB_PATH):
+        _build.build_library()
+    C = ctypes.CDLL(_build.CEILING_LIB_PATH)
+    C.tftq_ceiling_bytes.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                     ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)]
+    C.tftq_ceiling_launch.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                      ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    ws, rank, nsets = 8, 3, max(2, args.sets)
+    stream = torch.cuda.current_stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
+
+    def timed(launch, nbytes):
+        for i in range(args.warmup):
+            launch(i)
+        pairs = [(ev(), ev()) for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(pairs):
+            a.record(stream)
+            launch(i)
+            b.record(stream)
+        torch.cuda.synchronize()
+        us = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+        mean = sum(us) / len(us)
+        return {"us": round(mean, 2), "us_min": round(us[0], 2), "bytes": nbytes,
+                "GBs": round(nbytes / mean / 1e3, 1), "frac_of_peak": round(nbytes / mean / 1e3 / HBM_PEAK_GBS, 4)}
+
+    # footprint of benchmark configuration 3: 436 MB of bf16 tensors, 218 MB packed, slots of 27 MB
+    big = 13312 * 32768  # 436 207 616 bytes
+    rows, row_bytes = 6656, 4100  # one slot of 4096-column rows
+    slot = 27292672               # slot size of benchmark configuration 3 (a multiple of 128)
+    bufs = [(torch.empty(big, dtype=torch.uint8, device=dev).random_(),
+             torch.empty(big, dtype=torch.uint8, device=dev).random_()) for _ in range(nsets)]
+    NT, PLAIN = (1,), (0,)
+    BOTH = (0, 1)
+    # (label, kind, units, eighths, nt_loads choices, nt_stores choices)
+    kinds = [("read only", 0, 13312, 0, BOTH, PLAIN), ("write only", 1, 13312, 0, PLAIN, BOTH),
+             ("2:1 read:write (quantize, 16-bit tensors)", 2, 13312, 0, BOTH, BOTH),
+             ("1:2 read:write (dequantize, 16-bit tensors)", 3, 13312, 0, BOTH, BOTH),
+             ("4:1 read:write (quantize, fp32 tensors)", 4, 13312, 0, BOTH, BOTH),
+             ("1:4 read:write (dequantize, fp32 tensors)", 5, 13312, 0, BOTH, BOTH),
+             ("8:1 read:write, one contiguous source (reduce, 8 peers)", 6, 6656, 0, BOTH, BOTH),
+             ("reduce's accesses: 8 slots, 4100-byte rows, in place, an eighth of the rows per XCD",
+              7, rows, 1, NT, PLAIN),
+             ("reduce's accesses, rows in workgroup order", 7, rows, 0, NT, PLAIN),
+             ("reduce's accesses, an eighth per XCD, wavefronts start on 128-byte lines", 8, rows, 1, NT, PLAIN),
+             ("dequantize's accesses: 4100-byte packed rows -> 8 KB rows, rows in workgroup order",
+              9, 8 * rows, 0, NT, NT),
+             ("dequantize's accesses, an eighth of the rows per XCD", 9, 8 * rows, 1, NT, NT)]
+    ceilings = {}
+    for name, kind, units, eighths, ntls, ntss in kinds:
+        rb, wb = ctypes.c_int64(), ctypes.c_int64()
+        assert C.tftq_ceiling_bytes(kind, units, row_bytes, ctypes.byref(rb), ctypes.byref(wb)) == 0
+        for ntl in ntls:
+            for nts in ntss:
+                def launch(i, kind=kind, units=units, eighths=eighths, ntl=ntl, nts=nts):
+                    a, b = bufs[i % nsets]
+                    rc = C.tftq_ceiling_launch(kind, a.data_ptr(), b.data_ptr(), units, slot, row_bytes,
+                                               rank, eighths, ntl, nts, sp)
+                    assert rc == 0, rc
+                label = name
+                if kind < 7:
+                    label += (", streaming loads" if ntl else ", plain loads") if rb.value else ""
+                    label += (", streaming stores" if nts else ", plain stores") if wb.value else ""
+                r = timed(launch, rb.value + wb.value)
+                r["read_bytes"], r["write_bytes"], r["kind"] = rb.value, wb.value, kind
+                ceilings[label] = r
+    del bufs
+
+    # the product kernels on benchmark configuration 3, each alone in the same kind of loop
+    sets = []
+    for k in range(nsets):
+        t = workloads.cfg3(1000 * k + rank, device=dev)
+        packed = q.fused_quantize_into_fp8(t, ws)
+        sets.append({"tensors": t, "recv": packed.clone(), "gathered": packed})
+    ab = workloads.algorithmic_bytes(sets[0]["tensors"], ws)
+    product = {
+        "quantize": timed(lambda i: q.fused_quantize_into_fp8(sets[i % nsets]["tensors"], ws), ab["quantize"]),
+        "reduce": timed(lambda i: q.fused_reduce_fp8(sets[i % nsets]["tensors"], sets[i % nsets]["recv"], ws,
+                                                     rank, ReduceOp.AVG), ab["reduce"]),
+        "dequantize": timed(lambda i: q.fused_dequantize_from_fp8(sets[i % nsets]["tensors"],
+                                                                  sets[i % nsets]["gathered"], ws), ab["dequantize"]),
+    }
+
+    def best(kind):
+        return max((v for v in ceilings.values() if v["kind"] == kind), key=lambda v: v["GBs"])
+
+    mix = {"quantize": 2, "reduce": 6, "dequantize": 3}
+    for stage, kind in mix.items():
+        c = best(kind)
+        product[stage]["ceiling_GBs"] = c["GBs"]
+        product[stage]["of_ceiling"] = round(product[stage]["GBs"] / c["GBs"], 4)
+    for stage, kind in (("reduce", 7), ("dequantize", 9)):
+        c = best(kind)
+        product[stage]["own_accesses_GBs"] = c["GBs"]
+        product[stage]["of_own_accesses"] = round(product[stage]["GBs"] / c["GBs"], 4)
+    out = {"metric": "streaming ceilings and product kernels, each kernel alone, HBM GB/s on 1 MI355X",
+           "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "config": {"workload": "footprint of benchmark configuration 3 (436 MB of 16-bit tensors, 218 MB "
+                                  f"packed, 8 slots); {nsets} rotating buffer sets"},
+           "ceilings": ceilings, "product": product}
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the quantized-collective kernels run on one GPU's share "
               "and this build has no cross-GPU path; run with --gpus 1", file=sys.stderr)
         return 2
+    if args.config == "ceiling":
+        import torch
+        from torchft_amd import _lib
+        if not torch.cuda.is_available() or _lib.load().tftq_check_device() != 0:
+            print("bench.py needs a gfx950 GPU", file=sys.stderr)
+            return 2
+        return run_ceilings(args)
 
     import torch
     from torch.distributed import ReduceOp

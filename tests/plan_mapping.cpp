@@ -28,7 +28,7 @@ static uint32_t rnd()
 // (segment, workgroup number) of workgroup id b, or false when b has no work
 static bool locate_inline(const tftq_plan *p, int st, uint32_t b, int *seg, int *vb)
 {
-    const int x = (int)(b & 7), i = (int)(b >> 3);
+    const int x = (int)(b & 7), i = p->natural[st] ? (int)b : (int)(b >> 3);
     const Dealt &d = p->dealt[st];
     int base = d.base[x][0], sg = d.seg[x][0];
     for (int j = 1; j < TFTQ_N_INLINE; j++)
@@ -109,13 +109,7 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
             const Seg &s = p->segs[(size_t)i];
             const int64_t m_pad = (int64_t)s.slice_rows * ws;
             const int64_t rows = st == ST_Q ? m_pad : st == ST_R ? s.slice_rows : s.m;
-            int per_wg;
-            if (s.kind[st] == K_COL1) per_wg = tftq_col1_rows_per_wg(st);
-            else if (s.kind[st] == K_VECS) per_wg = tftq_small_rows_per_wg(s.n / (dtype == TFTQ_F32 ? 4 : 8));
-            else {
-                const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
-                per_wg = st == ST_R ? teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws) : teams;
-            }
+            const int per_wg = tftq_rows_per_wg(s, st, dtype == TFTQ_F32 ? 4 : 2, ws);
             const int64_t blocks = (rows + per_wg - 1) / per_wg;
             seen[(size_t)i].assign((size_t)blocks, 0);
             total += blocks;

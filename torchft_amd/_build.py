@@ -12,6 +12,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libtftq.so")
 SOURCES = ["tftq_quantize.hip", "tftq_reduce.hip", "tftq_dequantize.hip", "tftq_plan.cpp"]
+# Streaming kernels without arithmetic that bench.py times beside the product kernels
+# (benchmark infrastructure; torchft_amd never loads this library).
+CEILING_LIB_PATH = os.path.join(_HERE, "libtftq_ceiling.so")
+CEILING_SOURCE = "tftq_ceiling.hip"
 
 # -ffp-contract=off: the arithmetic contract is separate IEEE multiply, divide
 # and add; fused multiply-adds are written out where they are wanted.
@@ -47,6 +51,7 @@ def build_library(verbose: bool = False) -> str:
     with tempfile.TemporaryDirectory(prefix="tftq_build_") as tmp:
         objs = [os.path.join(tmp, os.path.splitext(s)[0] + ".o") for s in SOURCES]
         cmds = [[hipcc, *HIPCC_FLAGS, "-c", "-o", o, os.path.join(CSRC, s)] for s, o in zip(SOURCES, objs)]
+        cmds.append([hipcc, *HIPCC_FLAGS, "-shared", "-o", CEILING_LIB_PATH, os.path.join(CSRC, CEILING_SOURCE)])
         with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
             outs = list(pool.map(_run, cmds))
         outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]))

@@ -25,6 +25,7 @@ DEV bool rows_fill_lines(const Seg &s)
 template <typename T, bool POST>
 DEV float fin(float v, const KParams &p)
 {
+
     return POST ? Elem<T>::rounded(v) * p.post_scale : v;
 }
 
@@ -52,29 +53,20 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
-// Contiguous, 16-byte aligned rows.  Four vectors per lane and step; their loads
-// are issued together without a branch (lanes past the end re-read the last
-// vector and do not store).
+// Contiguous rows.  DV vectors per lane and step; their loads are issued together
+// without a branch (lanes past the end re-read the last vector and do not store),
+// and the first step's loads are on their way before the row's scale has arrived
+// and been turned into division coefficients.
 template <typename T, int TEAM, bool NT, int DV, bool POST>
 DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
 {
     if (row >= s.m) return;
     GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
-    const DivCoef c = make_div(as_f(in[0]));
-    if (!c.fast) {  // same for all lanes of the team
-        dequantize_gen<T, TEAM, POST>(s, p, row, lane);
-        return;
-    }
     constexpr int EPV = Elem<T>::EPV;
     const int nvec = s.n / EPV;
-    GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
-    // the few columns after the last whole vector, one element per lane
-    for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
-        const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
-        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p));
-    }
-    for (int base = 0; base < nvec; base += DV * TEAM) {
-        u32x2 w[DV];
+    const float sraw = as_f(in[0]);
+    u32x2 w[DV];
+    auto load_step = [&](int base) {
 #pragma unroll
         for (int k = 0; k < DV; k++) {
             const int idx = min(base + k * TEAM + lane, nvec - 1);
@@ -85,6 +77,20 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
                 w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
             }
         }
+    };
+    load_step(0);
+    const DivCoef c = make_div(sraw);
+    if (!c.fast) {  // same for all lanes of the team
+        dequantize_gen<T, TEAM, POST>(s, p, row, lane);
+        return;
+    }
+    GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
+    // the few columns after the last whole vector, one element per lane
+    for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
+        const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
+        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p));
+    }
+    for (int base = 0;;) {
 #pragma unroll
         for (int k = 0; k < DV; k++) {
             const int idx = base + k * TEAM + lane;
@@ -103,6 +109,9 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
                 else out[idx] = Elem<T>::pack(o);
             }
         }
+        base += DV * TEAM;
+        if (base >= nvec) break;
+        load_step(base);
     }
 }
 

@@ -171,6 +171,7 @@ DEV float div_fast(float f, float r, float r_lo) { return __builtin_fmaf(f, r, f
 // stored result of dequantize can.
 DEV float div_fast_signed(float f, float r, float r_lo)
 {
+
     return __builtin_copysignf(div_fast(f, r, r_lo), f);
 }
 
@@ -350,8 +351,9 @@ template <bool INLINE, int STAGE>
 DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
 {
     const int x = (int)(blockIdx.x & 7);
-    const int i = (int)(blockIdx.x >> 3);
+    int i = (int)(blockIdx.x >> 3);
     if (INLINE) {
+        if (p.natural) i = (int)blockIdx.x;  // all eight rows of the table describe the whole work
         // One round of scalar loads fetches this XCD's three table rows; the position
         // is then found in registers, and only the segment descriptor needs a second round.
         const CONSTANT char *karg = (const CONSTANT char *)__builtin_amdgcn_kernarg_segment_ptr();
@@ -449,10 +451,12 @@ static inline void work_mapping(const tftq_plan *plan, int stage, KParams *kp)
     if (plan->nseg <= TFTQ_N_INLINE) {
         kp->dealt = plan->dealt[stage];
         kp->per_xcd = plan->dealt_per_xcd[stage];
+        kp->natural = plan->natural[stage] ? 1 : 0;
         kp->map_shift = kp->chunk_shift = 0;
         kp->sorted_off = kp->map_off = 0;
     } else {
         kp->per_xcd = plan->index[stage].per_xcd;
+        kp->natural = 0;
         kp->map_shift = plan->index[stage].shift;
         kp->chunk_shift = plan->index[stage].chunk_shift;
         kp->sorted_off = plan->index[stage].sorted_off;

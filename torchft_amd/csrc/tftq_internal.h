@@ -131,6 +131,16 @@ struct Seg {
 };
 static_assert(sizeof(Seg) == 64, "Seg must be 64 bytes");
 
+// Rows of segment s that one workgroup takes in a stage.
+static inline int tftq_rows_per_wg(const Seg &s, int st, int esz, int ws)
+{
+    if (s.kind[st] == K_COL1) return tftq_col1_rows_per_wg(st);
+    if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
+    const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
+    if (st == ST_R) return teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws);
+    return teams;
+}
+
 struct InlineTable {
     Seg s[TFTQ_N_INLINE];
 };
@@ -180,6 +190,7 @@ struct tftq_plan {
     bool parked;               // quantize: some row also needs the 60 KB of LDS (rows above TFTQ_Q_VECS_WIDE)
     Dealt dealt[3];            // inline table only
     int32_t dealt_per_xcd[3];  // inline table only: workgroups of the busiest XCD
+    bool natural[3];           // inline table only: workgroup ids keep their order (see deal_to_xcds)
     TableIndex index[3];       // device table only
     std::vector<Seg> segs;
     std::vector<uint8_t> blob;  // host image of the device table (nseg > TFTQ_N_INLINE)
@@ -196,6 +207,7 @@ struct KParams {
     int32_t ws;
     int32_t rank;
     int32_t per_xcd;    // workgroup ids per XCD in the grid
+    int32_t natural;    // inline table only: workgroup id b is piece b of the work, not piece b / 8 of XCD b % 8
     int32_t map_shift;  // device table only, as are the next three
     int32_t chunk_shift;
     int64_t sorted_off;

@@ -93,19 +93,10 @@ static uint8_t pick_reduce_kind(const Seg &s)
     return K_GEN256;
 }
 
-static int rows_per_wg_of(const Seg &s, int st, int esz, int ws)
-{
-    if (s.kind[st] == K_COL1) return tftq_col1_rows_per_wg(st);
-    if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
-    const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
-    if (st == ST_R) return teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws);
-    return teams;
-}
-
 // Bytes one workgroup of segment s moves in a stage.
 static double wg_weight(const Seg &s, int st, int esz, int ws)
 {
-    const double rows = (double)rows_per_wg_of(s, st, esz, ws);
+    const double rows = (double)tftq_rows_per_wg(s, st, esz, ws);
     if (st == ST_R) return rows * (double)s.row_bytes * (ws + 1);
     return rows * ((double)s.n * esz + (double)s.row_bytes);
 }
@@ -127,6 +118,31 @@ static void work_order(const tftq_plan *p, int st, std::vector<int32_t> &ord)
     std::stable_sort(ord.begin(), ord.end(), [&](int32_t a, int32_t b) { return w[(size_t)a] > w[(size_t)b]; });
 }
 
+// Whether a stage hands its workgroups to the XCDs in their natural order (workgroup id b is
+// piece b of the work: neighbouring pieces run on different XCDs at the same time and the
+// whole chip works on one compact window of memory) instead of a contiguous eighth per XCD.
+// Measured on MI355X, kernel sequences on 218 M elements: dequantize is 1 to 6 % faster in
+// natural order (4096 bf16 columns 122.0 -> 117.9 us, 14336: 122.4 -> 115.7, 256: 148.0 ->
+// 140.4, 4096 fp32: 101.4 -> 96.3) when the tensor rows are whole 64-byte blocks, and 5 %
+// slower when they are not (1000 columns: neighbouring rows then share blocks across XCDs);
+// quantize gains 2.5 % for fp32 tensors and loses up to 2 % for 16-bit ones; reduce does not care
+// and keeps the eighths, which its heaviest-first order is built on.
+static bool natural_order(const tftq_plan *p, int st)
+{
+    if (st == ST_R || (st == ST_Q && p->esz != 4)) return false;
+    double whole = 0.0, all = 0.0;
+    for (int i = 0; i < p->nseg; i++) {
+        const Seg &s = p->segs[(size_t)i];
+        const double bytes = (double)s.m * (double)s.n * p->esz;
+        const bool fills = s.n == 1 ? s.row_stride == 1
+                                    : s.col_stride == 1 && ((int64_t)s.n * p->esz) % 64 == 0 &&
+                                          (s.row_stride * p->esz) % 64 == 0;
+        all += bytes;
+        if (fills) whole += bytes;
+    }
+    return whole * 2.0 >= all && all > 0.0;
+}
+
 // Few segments (the table travels in the kernel arguments).  Workgroup ids are
 // dealt round-robin to the 8 XCDs by the hardware; here every XCD takes a
 // contiguous eighth of every segment, so all XCDs see the same mix of row
@@ -143,6 +159,7 @@ static void deal_to_xcds(tftq_plan *p, const int32_t (*wgs)[3])
         work_order(p, st, ord);
         Dealt &d = p->dealt[st];
         int64_t busiest = 0;
+        p->natural[st] = natural_order(p, st);
         for (int x = 0; x < 8; x++) {
             int64_t cum = 0;
             for (int k = 0; k < TFTQ_N_INLINE; k++) {
@@ -154,8 +171,9 @@ static void deal_to_xcds(tftq_plan *p, const int32_t (*wgs)[3])
                 }
                 const int i = ord[(size_t)k];
                 const uint64_t n = (uint64_t)wgs[i][st];
-                const int64_t lo = (int64_t)((n * (uint64_t)x) >> 3);
-                const int64_t hi = (int64_t)((n * (uint64_t)(x + 1)) >> 3);
+                // natural order: every row of the table covers all workgroups of every segment
+                const int64_t lo = p->natural[st] ? 0 : (int64_t)((n * (uint64_t)x) >> 3);
+                const int64_t hi = p->natural[st] ? (int64_t)n : (int64_t)((n * (uint64_t)(x + 1)) >> 3);
                 d.base[x][k] = (int32_t)(p->segs[(size_t)i].wg_begin[st] + lo - cum);
                 d.seg[x][k] = i;
                 cum += hi - lo;
@@ -163,7 +181,7 @@ static void deal_to_xcds(tftq_plan *p, const int32_t (*wgs)[3])
             }
             if (cum > busiest) busiest = cum;
         }
-        p->dealt_per_xcd[st] = (int32_t)busiest;
+        p->dealt_per_xcd[st] = (int32_t)(p->natural[st] ? (busiest + 7) / 8 : busiest);
     }
 }
 
@@ -280,7 +298,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
         s.kind[ST_R] = pick_reduce_kind(s);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
-            const int64_t n = cdiv64(rows[st], rows_per_wg_of(s, st, p->esz, ws));
+            const int64_t n = cdiv64(rows[st], tftq_rows_per_wg(s, st, p->esz, ws));
             wgs[i][st] = (int32_t)n;
             wg[st] += n;
             if (wg[st] > INT32_MAX - 4096) {
@@ -292,6 +310,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
     for (int st = 0; st < 3; st++) p->nwg[st] = (int32_t)wg[st];
     p->wide[ST_Q] = p->wide[ST_R] = p->wide[ST_D] = false;
     p->parked = false;
+    p->natural[ST_Q] = p->natural[ST_R] = p->natural[ST_D] = false;
     for (int i = 0; i < n_tensors; i++) {
         const Seg &s = p->segs[(size_t)i];
         const int nvec = s.n / (16 / p->esz), ndw = s.row_bytes / 4 - 1;
