@@ -35,6 +35,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch on benchmark configuration 3 as profiled (profiles/cfg3_bf16_ws8_hbm_traffic.md)
+PROFILED_TRAFFIC = {"quantize": 655142000, "reduce": 246760000, "dequantize": 661483000}
 
 
 def parse_args():
@@ -427,6 +429,33 @@ def main() -> int:
     torch.cuda.synchronize()
     stage_ms = stage_means(all_events, range(3))
 
+    # Every stage alone: K launches of the one kernel, rotating over the buffer sets, events
+    # around each launch (not part of the timed region).  In a quantized all-reduce the kernels
+    # never run back to back (collectives lie between them, torchft/collectives.py:364-412); in the
+    # step above a kernel also pays for the write-back of what the one before it left in the
+    # caches, here it does not.
+    def alone(k, i):
+        s = sets[i % len(sets)]
+        if k == 0:
+            q.fused_quantize_into_fp8(s["tensors"], ws)
+        elif k == 1:
+            q.fused_reduce_fp8(s["tensors"], s["recv"], ws, rank, op)
+        else:
+            q.fused_dequantize_from_fp8(s["tensors"], s["gathered"], ws)
+
+    alone_ms = {}
+    stream = torch.cuda.current_stream()
+    for k in range(3):
+        for i in range(args.warmup):
+            alone(k, i)
+        pairs = [(ev(), ev()) for _ in range(args.steps)]
+        for i, (a, b) in enumerate(pairs):
+            a.record(stream)
+            alone(k, i)
+            b.record(stream)
+        torch.cuda.synchronize()
+        alone_ms[STAGES[k]] = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+
     total_bytes = sum(ab.values())
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -436,16 +465,28 @@ def main() -> int:
         stages[k] = {"us": round(stage_ms[k] * 1e3, 2), "bytes": ab[k], "GBs": round(gbs, 1),
                      "frac": round(gbs / HBM_PEAK_GBS, 4)}
     stages["note"] = "separate pass with events around every stage; the timed region has events around the dominant kernel only"
+    stages_alone = {}
+    for k in alone_ms:
+        gbs = ab[k] / (alone_ms[k] * 1e-3) / 1e9
+        stages_alone[k] = {"us": round(alone_ms[k] * 1e3, 2), "GBs": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    stages_alone["note"] = ("each kernel alone in a loop over the buffer sets, events around every launch "
+                            "(an event pair adds 2-3 us to the kernel's own duration)")
 
-    # The roofline entry is for the kernel that takes the largest share of the step.
-    # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE (x2.000,
-    # calibrated on a 256 MiB copy) + WRITE_SIZE (x1.000); profiles/cfg3_bf16_ws8_hbm_traffic.md
-    measured_traffic = {"quantize": 655142000, "reduce": 246760000, "dequantize": 661483000}
+    # The roofline entry is for the kernel that takes the largest share of the step: HIP events
+    # around its launches inside the timed region (they include the gap to the kernel before it).
+    # `traffic` is not measured by this run: HBM bytes per launch on the headline workload from
+    # rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated on a 256 MiB copy) + WRITE_SIZE (x1.000), as
+    # recorded in profiles/cfg3_bf16_ws8_hbm_traffic.md.
+    profiled_traffic = PROFILED_TRAFFIC if args.config == "3" else {}
     achieved = ab[dominant] / (dominant_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "k_" + dominant, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "us": round(dominant_ms * 1e3, 2),
-                "traffic": measured_traffic[dominant] if args.config == "3" else None}
+                "timing": "HIP events around the kernel inside the timed quantize -> reduce -> dequantize steps",
+                "alone": stages_alone[dominant],
+                "traffic": profiled_traffic.get(dominant),
+                "traffic_source": "profiles/cfg3_bf16_ws8_hbm_traffic.md (rocprofv3 --pmc, not this run)"
+                                  if profiled_traffic else None}
 
     out = {
         "metric": "quantize+reduce+dequant HBM GB/s on 1 MI355X",
@@ -467,6 +508,7 @@ def main() -> int:
                    "algorithmic_bytes_per_step": total_bytes},
         "roofline": roofline,
         "stages": stages,
+        "stages_alone": stages_alone,
         "parity": "quantize, reduce, dequantize byte-identical to the CPU checker on the probe tensor",
     }
     if not args.no_cpu_baseline and args.config == "3":

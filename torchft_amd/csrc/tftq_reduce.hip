@@ -536,6 +536,85 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
     }
 }
 
+// One row per team with UNITS >= 2 vectors per lane and peer, as a rolling window over the
+// peers: as soon as a lane has taken vector u of peer k out of its registers, the load of
+// vector u of peer k + 1 is issued into them, so UNITS loads are in flight all the time at
+// the register cost of one peer.  The last peer is peeled off: nothing is loaded behind it.
+// Same requirements as reduce_rows.
+template <int TEAM, int UNITS, bool GDIV>
+DEV void reduce_rows_roll(const Seg &s, const KParams &p, int j, int lane, float *lds)
+{
+    const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
+    const int ws = p.ws;
+    const int wlane = TEAM >= 64 ? (int)(threadIdx.x & 63u) : lane;
+    const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+
+    u32 boff[UNITS];     // byte offset of vector u of this lane in the payload (see reduce_rows)
+    u32 padmask[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        const int d = min(4 * (u * TEAM + lane), ndw - 4);
+        boff[u] = 4u * (u32)d;
+        padmask[u] = (d == ndw - 4 && (s.n & 3)) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+    }
+    const float raw_scale = as_f(peer_row(p, speer, off)[0]);
+    u32x4 w[UNITS];
+    {
+        GLOBAL const uint8_t *pv = (GLOBAL const uint8_t *)(peer_row(p, 0, off) + 1);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + boff[u]));
+    }
+    float acc[UNITS][16];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+    const float sc = raw_scale == 0.0f ? 1.0f : raw_scale;  // padding rows (:419)
+    const DivCoef c = make_div(sc);
+    const bool row_fast = __builtin_amdgcn_ballot_w64(!c.fast) == 0;  // same in all wavefronts of the team
+    if (row_fast) {
+#pragma nounroll
+        for (int k = 0; k + 1 < ws; k++) {
+            const float pr = team_bcast<TEAM>(c.r, k), pl = team_bcast<TEAM>(c.r_lo, k);
+            GLOBAL const uint8_t *pv = (GLOBAL const uint8_t *)(peer_row(p, k + 1, off) + 1);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                u32x4 x = w[u];
+                asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // taken out before the registers are loaded again
+                w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + boff[u]));
+                x.w &= padmask[u];
+                accumulate16(acc[u], x, pr, pl);
+            }
+        }
+        {
+            const float pr = team_bcast<TEAM>(c.r, ws - 1), pl = team_bcast<TEAM>(c.r_lo, ws - 1);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                u32x4 x = w[u];
+                x.w &= padmask[u];
+                accumulate16(acc[u], x, pr, pl);
+            }
+        }
+        float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
+#pragma unroll
+        for (int u = 0; u < UNITS; u++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+        amax = team_max<TEAM>(amax, lds);
+        const float s2 = calc_scale(amax_div<GDIV>(amax, p));  // :340
+        GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            const u32x4 o = requant16<GDIV>(acc[u], s2, p);
+            if (4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)((GLOBAL uint8_t *)(orow + 1) + boff[u]) = o;
+        }
+        if (lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+    } else {
+        reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
+    }
+}
+
 // Few peers (ws <= 4): ROWS consecutive rows of one team at once, all loads of
 // all rows issued together, so that a lane has 8 vectors in flight although a
 // row has only ws * UNITS of them.  ws * UNITS * ROWS <= 8.  Rows past the end of
@@ -730,12 +809,22 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         } else if (p.ws > 64) {
             if (ndw <= 1024) reduce_row<256, 1, GDIV>(s, p, j, tid, lds);
             else reduce_row<256, 4, GDIV>(s, p, j, tid, lds);
-        } else if (ndw <= 1024) {
-            reduce_rows<256, 1, true, GDIV>(s, p, j, tid, lds);
-        } else if (ndw <= 2048) {
-            reduce_rows<256, 2, true, GDIV>(s, p, j, tid, lds);
         } else {
-            reduce_rows<256, 4, false, GDIV>(s, p, j, tid, lds);
+            // Vectors per lane and peer that this wavefront needs: lane l of the team holds
+            // dwords 4 * (256 * u + l) ..., so the upper wavefronts of a row whose length is
+            // not a multiple of 1024 dwords need one vector less than the lower ones
+            // (10240 columns: 3, 3, 2, 2 instead of 3 each: 55.0 -> 50.4 us on [20480, 10240]).
+            // Every variant passes the team's barriers the same number of times.
+            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+            const int nu = min((ndw + 1023) >> 10, (ndw - 256 * wave + 1023) >> 10);
+            if (nu == 1) reduce_rows<256, 1, true, GDIV>(s, p, j, tid, lds);
+            // rows of three or four vectors per lane run the rolling window in all their wavefronts
+            // ([20480, 10240]: 53.5 -> 50.4 us against the pipeline in the upper two); rows of two
+            // are faster in the pipeline (5120 columns: 50.9 against 62.1 us)
+            else if (nu == 2 && ndw > 2048) reduce_rows_roll<256, 2, GDIV>(s, p, j, tid, lds);
+            else if (nu == 2) reduce_rows<256, 2, true, GDIV>(s, p, j, tid, lds);
+            else if (nu == 3) reduce_rows_roll<256, 3, GDIV>(s, p, j, tid, lds);
+            else reduce_rows_roll<256, 4, GDIV>(s, p, j, tid, lds);
         }
         break;
     }
