@@ -269,7 +269,7 @@ def main() -> int:
     if args.config == "ceiling":
         import torch
         from torchft_amd import _lib
-        if not torch.cuda.is_available() or _lib.load().tftq_check_device() != 0:
+        if not torch.cuda.is_available() or _lib.load().tftq_check_device(0) != 0:
             print("bench.py needs a gfx950 GPU", file=sys.stderr)
             return 2
         return run_ceilings(args)
@@ -284,7 +284,7 @@ def main() -> int:
         print("bench.py needs a gfx950 GPU", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
-    rc = _lib.load().tftq_check_device()
+    rc = _lib.load().tftq_check_device(0)
     if rc != 0:
         print("bench.py: " + _lib.strerror(rc), file=sys.stderr)
         return 2

@@ -10,11 +10,21 @@
  * Conventions
  *  - every function returns 0 on success; a negative value is a TFTQ_E_* code,
  *    a positive value is a hipError_t.  Nothing aborts or throws.
- *  - device pointers must belong to the device that is current on the calling
- *    thread; kernels are enqueued on `stream` (a hipStream_t passed as void*,
- *    NULL = the null stream) and the host is never synchronised.
- *  - functions are thread-safe; a plan may be used from several threads at
- *    once (it is immutable after tftq_plan_set_device_table).
+ *  - a plan describes shapes, strides, element type and group size only.  It
+ *    holds no address and belongs to no device: tensor addresses, the packed
+ *    buffer, the device and the stream are arguments of every compute call.
+ *  - `device` is the ordinal of the device that all device addresses of the
+ *    call belong to; the library makes it current for the duration of the
+ *    call and restores the caller's device before it returns.  -1 = the device
+ *    that is current on the calling thread.
+ *  - kernels are enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *    null stream) and the host is never synchronised.
+ *  - functions are thread-safe; a plan is immutable and may be used from
+ *    several threads, devices and streams at once.
+ *  - the library allocates no device memory.  Lists of up to TFTQ_N_INLINE
+ *    tensors need none beyond tensors and packed buffer (their descriptors
+ *    travel in the kernel arguments); longer lists need two caller-owned device
+ *    buffers, see "Long lists" below.
  *
  * Packed buffer (byte-for-byte the reference's, quantization.py:108-123,
  * 495-503), for tensor i of shape [m_i, n_i] and group size ws:
@@ -37,12 +47,15 @@
 extern "C" {
 #endif
 
-#define TFTQ_VERSION 1
+#define TFTQ_VERSION 2
 
 /* element types of the tensors being (de)quantized (quantization.py:474-478) */
 #define TFTQ_F32 0
 #define TFTQ_F16 1
 #define TFTQ_BF16 2
+
+/* lists of at most this many tensors need no device memory for their descriptors */
+#define TFTQ_N_INLINE 16
 
 /* error codes (negative); positive return values are hipError_t */
 #define TFTQ_E_ARG (-1)      /* bad argument (null pointer, ws <= 0, rank out of range ...) */
@@ -50,20 +63,24 @@ extern "C" {
 #define TFTQ_E_SHAPE (-3)    /* negative or too large dimension */
 #define TFTQ_E_SIZE (-4)     /* "Output size does not match" (:621, :672) */
 #define TFTQ_E_NOMEM (-5)    /* host allocation failed */
-#define TFTQ_E_NOTABLE (-6)  /* plan needs a device table that was not provided */
-#define TFTQ_E_ARCH (-7)     /* current device is not gfx950 */
+#define TFTQ_E_NOTABLE (-6)  /* a list longer than TFTQ_N_INLINE needs `table` (and `pointers`) */
+#define TFTQ_E_ARCH (-7)     /* the device is not gfx950 */
 
 typedef struct tftq_plan tftq_plan;
 
 /* library version (TFTQ_VERSION of the build) */
 int tftq_version(void);
 
+/* Identifies the sources the library was built from (a hash that the build passes in;
+ * "unknown" without one).  Static storage. */
+const char *tftq_build_id(void);
+
 /* Text for a return value of this library (static storage). */
 const char *tftq_strerror(int code);
 
-/* 0 when the current device can run the kernels (gfx950), else TFTQ_E_ARCH or
- * a hipError_t. */
-int tftq_check_device(void);
+/* 0 when device `device` (-1: the current one) can run the kernels (gfx950), else
+ * TFTQ_E_ARCH or a hipError_t. */
+int tftq_check_device(int device);
 
 /*
  * Layout arithmetic of _prepare_quantize_fp8 (quantization.py:486-503), host
@@ -76,58 +93,74 @@ int tftq_layout(int n_tensors, const int64_t *shapes, int ws, int64_t *slot_off,
 /*
  * Builds the work plan for one list of tensors: the layout above plus the
  * partition of all rows into workgroups for the three kernels.  Replaces the
- * four device tables that _prepare_quantize_fp8 uploads on every call
- * (quantization.py:505-515).  Host only, no HIP call.
+ * shape, stride and offset tables that _prepare_quantize_fp8 uploads on every
+ * call (quantization.py:505-515); the addresses (its fourth table) are an
+ * argument of the compute calls.  Host only, no HIP call.
  *   dtype    TFTQ_F32 / TFTQ_F16 / TFTQ_BF16
- *   ptrs     [n_tensors] device address of element (0,0) of each tensor; may
- *            be NULL for a plan that is only used with tftq_reduce
  *   shapes   [n_tensors][2] (m, n)
  *   strides  [n_tensors][2] element strides (row, column); any values
  */
-int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
-                     const int64_t *shapes, const int64_t *strides, int ws,
-                     tftq_plan **out);
+int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes, const int64_t *strides,
+                     int ws, tftq_plan **out);
 void tftq_plan_destroy(tftq_plan *plan);
 
 int64_t tftq_plan_output_size(const tftq_plan *plan); /* bytes of the packed buffer */
 int64_t tftq_plan_slot_size(const tftq_plan *plan);   /* output_size / ws */
 int64_t tftq_plan_max_rows(const tftq_plan *plan);    /* i_max_row_num of the reference */
+int tftq_plan_n_tensors(const tftq_plan *plan);
 
 /*
- * Plans with few tensors carry their descriptors in the kernel arguments and
- * need no device memory: tftq_plan_table_bytes() returns 0.  Larger plans need
- * a device copy of the descriptor table: allocate tftq_plan_table_bytes()
- * bytes (256-byte aligned) on the device, copy tftq_plan_table_host() into it
- * and hand the address over with tftq_plan_set_device_table() before the first
- * compute call.  The library never allocates device memory.
+ * Long lists (more than TFTQ_N_INLINE tensors).  The kernels read the
+ * descriptors from device memory that the caller owns:
+ *   table     tftq_plan_table_bytes() bytes, 256-byte aligned, holding a copy of
+ *             tftq_plan_table_host(): descriptors and lookup index, no addresses.
+ *             The same image serves every device, stream and list of tensors of
+ *             these shapes; copy it once per device, any way you like, before
+ *             the first kernel that uses it runs.
+ *   pointers  8 * n_tensors bytes, 8-byte aligned: the tensors' addresses.  When a
+ *             compute call is given `tensors` (host array), it first writes them
+ *             here with small kernels on `stream` (the host array is read
+ *             before the call returns; nothing blocks); with tensors == NULL it
+ *             uses what `pointers` already holds.  One `pointers` buffer must
+ *             not be written by calls that overlap in time.
+ * For short lists both are ignored (pass NULL) and tftq_plan_table_bytes() is 0.
  */
 int64_t tftq_plan_table_bytes(const tftq_plan *plan);
 const void *tftq_plan_table_host(const tftq_plan *plan);
-int tftq_plan_set_device_table(tftq_plan *plan, const void *device_table);
+
+/* Writes the n_tensors addresses of `tensors` (host array) to `pointers` (device) on
+ * `stream`: what the compute calls do when they are given `tensors` for a long list. */
+int tftq_upload_pointers(const tftq_plan *plan, const void *const *tensors, void *pointers,
+                         int device, void *stream);
 
 /*
- * fused_quantize_into_fp8 (quantization.py:531-588).  Reads the plan's
- * tensors, writes every byte of packed[0 .. output_size): scales, codes, zero
- * padding and zero padding rows, so `packed` needs no prior memset (the
- * reference relies on torch.zeros, :567-571).  packed must be 4-byte aligned.
+ * fused_quantize_into_fp8 (quantization.py:531-588).  Reads the tensors,
+ * writes every byte of packed[0 .. output_size): scales, codes, zero padding
+ * and zero padding rows, so `packed` needs no prior memset (the reference
+ * relies on torch.zeros, :567-571).  packed must be 4-byte aligned.
+ *   tensors  host array [n_tensors]: device address of element (0,0) of each
+ *            tensor (may be NULL for a long list whose `pointers` are current)
  */
-int tftq_quantize(const tftq_plan *plan, void *packed, int64_t packed_bytes, void *stream);
+int tftq_quantize(const tftq_plan *plan, const void *const *tensors, const void *table,
+                  void *pointers, void *packed, int64_t packed_bytes, int device, void *stream);
 
 /*
  * fused_reduce_fp8 (quantization.py:638-686).  packed holds ws slots, slot p =
  * peer p's quantization of this rank's row slice.  Sums the slots in fp32 in
  * the order rank, rank+1, ... (wrapping, :405-407), requantizes and overwrites
  * slot `rank` (scale and codes of every row, padding rows included).  is_avg
- * != 0 divides by ws (:682).  The plan's tensor pointers are not used.
+ * != 0 divides by ws (:682).  No tensor is touched (the reference's launcher
+ * ignores their addresses too, :675-686).
  */
-int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank,
-                int is_avg, void *stream);
+int tftq_reduce(const tftq_plan *plan, const void *table, void *packed, int64_t packed_bytes,
+                int rank, int is_avg, int device, void *stream);
 
 /*
  * fused_dequantize_from_fp8 (quantization.py:591-635).  Writes
- * cast(float(code) / scale) into the plan's tensors (all m_i real rows).
+ * cast(float(code) / scale) into the tensors (all m_i real rows).
  */
-int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
+int tftq_dequantize(const tftq_plan *plan, void *const *tensors, const void *table,
+                    void *pointers, const void *packed, int64_t packed_bytes, int device,
                     void *stream);
 
 /*
@@ -140,8 +173,9 @@ int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_by
  * computes with post_scale = (float)(1.0 / divisor).  The bytes equal those of
  * tftq_dequantize followed by that division.
  */
-int tftq_dequantize_scaled(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
-                           float post_scale, void *stream);
+int tftq_dequantize_scaled(const tftq_plan *plan, void *const *tensors, const void *table,
+                           void *pointers, const void *packed, int64_t packed_bytes,
+                           float post_scale, int device, void *stream);
 
 #ifdef __cplusplus
 }

@@ -81,14 +81,12 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
 {
     const int n = (int)shapes.size() / 2;
     std::vector<int64_t> strides((size_t)n * 2);
-    std::vector<const void *> ptrs((size_t)n);
     for (int i = 0; i < n; i++) {
         strides[2 * (size_t)i] = shapes[2 * (size_t)i + 1];
         strides[2 * (size_t)i + 1] = 1;
-        ptrs[(size_t)i] = (const void *)(uintptr_t)(0x10000 + 64 * (size_t)i);
     }
     tftq_plan *p = nullptr;
-    const int rc = tftq_plan_create(dtype, n, ptrs.data(), shapes.data(), strides.data(), ws, &p);
+    const int rc = tftq_plan_create(dtype, n, shapes.data(), strides.data(), ws, &p);
     if (rc) {
         printf("plan_create failed: %d\n", rc);
         return 1;

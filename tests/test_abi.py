@@ -23,7 +23,8 @@ def test_header_symbols_exported():
     for name in declared:
         assert hasattr(L, name), f"{name} declared in tftq.h but not exported"
     assert declared == {n for n, _, _ in _lib.SYMBOLS}
-    assert L.tftq_version() == 1
+    assert L.tftq_version() == 2
+    assert re.fullmatch(r"[0-9a-f]{16}|unknown", L.tftq_build_id().decode())
 
 
 def _layout(shapes, ws):
@@ -55,14 +56,13 @@ def test_layout_errors():
     assert _layout([(1, 2 ** 31)], 2)[0] == -3
 
 
-def _plan(dtype, shapes, strides, ws, ptrs=None):
+def _plan(dtype, shapes, strides, ws):
     L = _lib.load()
     T = len(shapes)
     sh = (ctypes.c_int64 * (2 * T))(*[v for s in shapes for v in s])
     st = (ctypes.c_int64 * (2 * T))(*[v for s in strides for v in s])
-    pp = (ctypes.c_void_p * T)(*(ptrs or [0x1000 * (i + 1) for i in range(T)]))
     h = ctypes.c_void_p()
-    rc = L.tftq_plan_create(dtype, T, pp, sh, st, ws, ctypes.byref(h))
+    rc = L.tftq_plan_create(dtype, T, sh, st, ws, ctypes.byref(h))
     return rc, h
 
 
@@ -82,10 +82,20 @@ def test_plan_sizes_and_table():
     assert L.tftq_plan_table_bytes(h) > 40 * 64 and L.tftq_plan_table_bytes(h) % 8 == 0
     assert L.tftq_plan_table_host(h)
     assert L.tftq_plan_max_rows(h) == 4
-    # no device table bound yet: compute entry points refuse instead of launching
+    assert L.tftq_plan_n_tensors(h) == 40
+    # the image holds no address: the first descriptor's pointer field is zero
+    assert ctypes.cast(L.tftq_plan_table_host(h), ctypes.POINTER(ctypes.c_uint64))[0] == 0
+    # without the device table the compute entry points refuse instead of launching
     buf = (ctypes.c_uint8 * L.tftq_plan_output_size(h))()
-    assert L.tftq_quantize(h, buf, len(buf), None) == -6
-    assert L.tftq_quantize(h, buf, len(buf) - 4, None) == -4
+    assert L.tftq_quantize(h, None, None, None, buf, len(buf), -1, None) == -6
+    assert L.tftq_reduce(h, None, buf, len(buf), 0, 0, -1, None) == -6
+    assert L.tftq_quantize(h, None, None, None, buf, len(buf) - 4, -1, None) == -4
+    L.tftq_plan_destroy(h)
+    # a short list needs its tensors' addresses
+    rc, h = _plan(2, [(8, 64)], [(64, 1)], 2)
+    buf = (ctypes.c_uint8 * L.tftq_plan_output_size(h))()
+    assert L.tftq_quantize(h, None, None, None, buf, len(buf), -1, None) == -1
+    assert L.tftq_quantize(h, (ctypes.c_void_p * 1)(None), None, None, buf, len(buf), -1, None) == -1
     L.tftq_plan_destroy(h)
 
 

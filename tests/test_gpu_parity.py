@@ -29,7 +29,7 @@ NT = min(16, os.cpu_count() or 1)
 def q():
     assert torch.cuda.is_available(), "GPU tests need a gfx950 device"
     from torchft_amd import _lib, quantization
-    assert _lib.load().tftq_check_device() == 0, "device is not gfx950"
+    assert _lib.load().tftq_check_device(0) == 0, "device is not gfx950"
     return quantization
 
 
@@ -665,18 +665,21 @@ def test_no_write_outside_packed_buffer(q):
     sh = (ctypes.c_int64 * (2 * T))(*[v for t in ts for v in t.shape])
     st = (ctypes.c_int64 * (2 * T))(*[v for t in ts for v in t.stride()])
     h = ctypes.c_void_p()
-    assert L.tftq_plan_create(2, T, ptrs, sh, st, ws, ctypes.byref(h)) == 0
+    assert L.tftq_plan_create(2, T, sh, st, ws, ctypes.byref(h)) == 0
     size = L.tftq_plan_output_size(h)
     arena = torch.full((size + 2 * guard,), 0xA5, dtype=torch.uint8, device="cuda")
     packed = arena[guard:guard + size]
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    assert L.tftq_quantize(h, ctypes.c_void_p(packed.data_ptr()), size, stream) == 0
-    assert L.tftq_reduce(h, ctypes.c_void_p(packed.data_ptr()), size, 1, 1, stream) == 0
-    assert L.tftq_dequantize(h, ctypes.c_void_p(packed.data_ptr()), size, stream) == 0
+    dev = torch.cuda.current_device()
+    p = ctypes.c_void_p(packed.data_ptr())
+    assert L.tftq_quantize(h, ptrs, None, None, p, size, dev, stream) == 0
+    assert L.tftq_reduce(h, None, p, size, 1, 1, dev, stream) == 0
+    assert L.tftq_dequantize(h, ptrs, None, None, p, size, -1, stream) == 0  # -1: the current device
     torch.cuda.synchronize()
     assert (arena[:guard] == 0xA5).all() and (arena[guard + size:] == 0xA5).all()
-    assert L.tftq_quantize(h, ctypes.c_void_p(packed.data_ptr()), size - 4, stream) == -4
-    assert L.tftq_reduce(h, ctypes.c_void_p(packed.data_ptr()), size, 4, 0, stream) == -1
+    assert L.tftq_quantize(h, ptrs, None, None, p, size - 4, dev, stream) == -4
+    assert L.tftq_reduce(h, None, p, size, 4, 0, dev, stream) == -1
+    assert L.tftq_quantize(h, None, None, None, p, size, dev, stream) == -1  # no addresses
     L.tftq_plan_destroy(h)
 
 
@@ -709,31 +712,35 @@ def test_entry_points_under_graph_capture(q, n_tensors):
     outs = [torch.empty_like(t) for t in ts]
     T = len(ts)
 
-    def plan_for(tensors):
-        ptrs = (ctypes.c_void_p * T)(*[t.data_ptr() for t in tensors])
-        sh = (ctypes.c_int64 * (2 * T))(*[v for t in tensors for v in t.shape])
-        st = (ctypes.c_int64 * (2 * T))(*[v for t in tensors for v in t.stride()])
-        h = ctypes.c_void_p()
-        assert L.tftq_plan_create(2, T, ptrs, sh, st, ws, ctypes.byref(h)) == 0
-        table = None
-        nbytes = L.tftq_plan_table_bytes(h)
-        if nbytes:
-            host = (ctypes.c_uint8 * nbytes).from_address(L.tftq_plan_table_host(h))
-            table = torch.frombuffer(host, dtype=torch.uint8).cuda()
-            assert L.tftq_plan_set_device_table(h, ctypes.c_void_p(table.data_ptr())) == 0
-        return h, table
-
-    h_in, keep_in = plan_for(ts)     # quantize and reduce read `ts`
-    h_out, keep_out = plan_for(outs)  # dequantize writes `outs`
-    size = L.tftq_plan_output_size(h_in)
+    # one plan (shapes only) serves both tensor lists; a list of 20 needs the device copy of
+    # the plan's table and a device buffer per list for the addresses
+    sh = (ctypes.c_int64 * (2 * T))(*[v for t in ts for v in t.shape])
+    st = (ctypes.c_int64 * (2 * T))(*[v for t in ts for v in t.stride()])
+    h = ctypes.c_void_p()
+    assert L.tftq_plan_create(2, T, sh, st, ws, ctypes.byref(h)) == 0
+    assert L.tftq_plan_n_tensors(h) == T
+    in_ptrs = (ctypes.c_void_p * T)(*[t.data_ptr() for t in ts])     # quantize reads `ts`
+    out_ptrs = (ctypes.c_void_p * T)(*[t.data_ptr() for t in outs])  # dequantize writes `outs`
+    table = in_dev = out_dev = None
+    nbytes = L.tftq_plan_table_bytes(h)
+    assert (nbytes > 0) == (T > 16)
+    if nbytes:
+        host = (ctypes.c_uint8 * nbytes).from_address(L.tftq_plan_table_host(h))
+        table = torch.frombuffer(host, dtype=torch.uint8).cuda()
+        in_dev = torch.empty(T, dtype=torch.int64, device="cuda")
+        out_dev = torch.empty(T, dtype=torch.int64, device="cuda")
+    size = L.tftq_plan_output_size(h)
     packed = torch.empty(size, dtype=torch.uint8, device="cuda")
+    dev = torch.cuda.current_device()
+    addr = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())  # noqa: E731
 
     def enqueue(stream):
         s = ctypes.c_void_p(stream.cuda_stream)
         p = ctypes.c_void_p(packed.data_ptr())
-        assert L.tftq_quantize(h_in, p, size, s) == 0
-        assert L.tftq_reduce(h_in, p, size, rank, 1, s) == 0
-        assert L.tftq_dequantize(h_out, p, size, s) == 0
+        # the addresses are written to the device buffers by small kernels that the capture records too
+        assert L.tftq_quantize(h, in_ptrs, addr(table), addr(in_dev), p, size, dev, s) == 0
+        assert L.tftq_reduce(h, addr(table), p, size, rank, 1, dev, s) == 0
+        assert L.tftq_dequantize(h, out_ptrs, addr(table), addr(out_dev), p, size, dev, s) == 0
 
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
@@ -763,8 +770,7 @@ def test_entry_points_under_graph_capture(q, n_tensors):
         same_bytes(got_packed, packed, f"replay {it}: packed buffer")
         for i, (a, b) in enumerate(zip(got, outs)):
             same_bytes(a, b, f"replay {it}: tensor {i}")
-    L.tftq_plan_destroy(h_in)
-    L.tftq_plan_destroy(h_out)
+    L.tftq_plan_destroy(h)
 
 
 @pytest.mark.parametrize("seed", range(int(os.environ.get("TFTQ_RANDOM_LISTS", "36"))))

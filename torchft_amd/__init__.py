@@ -2,9 +2,11 @@
 ``torchft.quantization`` (and its callers in ``torchft.collectives``)."""
 
 from .quantization import (  # noqa: F401
+    PreparedBucket,
     fused_dequantize_from_fp8,
     fused_quantize_into_fp8,
     fused_reduce_fp8,
+    prepare,
 )
 
 from .collectives import (  # noqa: F401
@@ -22,4 +24,6 @@ __all__ = [
     "fused_dequantize_from_fp8",
     "fused_quantize_into_fp8",
     "fused_reduce_fp8",
+    "prepare",
+    "PreparedBucket",
 ]

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import hashlib
 import os
 import shutil
 import subprocess
@@ -11,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libtftq.so")
-SOURCES = ["tftq_quantize.hip", "tftq_reduce.hip", "tftq_dequantize.hip", "tftq_plan.cpp"]
+SOURCES = ["tftq_quantize.hip", "tftq_reduce.hip", "tftq_dequantize.hip", "tftq_runtime.hip", "tftq_plan.cpp"]
 # Streaming kernels without arithmetic that bench.py times beside the product kernels
 # (benchmark infrastructure; torchft_amd never loads this library).
 CEILING_LIB_PATH = os.path.join(_HERE, "libtftq_ceiling.so")
@@ -26,6 +27,20 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
 ]
+
+
+def source_hash() -> str:
+    """Hash of everything libtftq.so is compiled from; the library reports the hash it was
+    built with as tftq_build_id()."""
+    h = hashlib.sha256()
+    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC))
+             if f.endswith((".hip", ".h", ".cpp")) and f != CEILING_SOURCE]
+    files.append(os.path.join(os.path.dirname(_HERE), "include", "tftq.h"))
+    for path in files:
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
 
 
 def hipcc_path() -> str:
@@ -50,7 +65,8 @@ def build_library(verbose: bool = False) -> str:
     hipcc = hipcc_path()
     with tempfile.TemporaryDirectory(prefix="tftq_build_") as tmp:
         objs = [os.path.join(tmp, os.path.splitext(s)[0] + ".o") for s in SOURCES]
-        cmds = [[hipcc, *HIPCC_FLAGS, "-c", "-o", o, os.path.join(CSRC, s)] for s, o in zip(SOURCES, objs)]
+        build_id = f'-DTFTQ_BUILD_ID="{source_hash()}"'
+        cmds = [[hipcc, *HIPCC_FLAGS, build_id, "-c", "-o", o, os.path.join(CSRC, s)] for s, o in zip(SOURCES, objs)]
         cmds.append([hipcc, *HIPCC_FLAGS, "-shared", "-o", CEILING_LIB_PATH, os.path.join(CSRC, CEILING_SOURCE)])
         with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
             outs = list(pool.map(_run, cmds))

@@ -35,6 +35,7 @@ import torch
 from torch.distributed import ReduceOp
 from torch.distributed.distributed_c10d import AllreduceOptions
 
+from . import quantization as _q
 from .collectives import allreduce_quantized
 
 
@@ -109,6 +110,7 @@ def allreduce(
     should_quantize: bool = False,
     reduce_op: ReduceOp = ReduceOp.AVG,
     fold_normalization: bool = True,
+    prepared: "_q.PreparedBucket | None" = None,
 ):
     """
     All-reduce ``tensor`` in place over ``process_group`` and scale it by
@@ -116,6 +118,9 @@ def allreduce(
     With ``should_quantize`` the scaling is part of the dequantize kernel unless
     ``fold_normalization`` is False (then it is a separate in-place division in
     the continuation, as in the reference); the resulting bytes are the same.
+
+    ``prepared``: ``torchft_amd.quantization.prepare([tensor], process_group.size())`` made
+    once for a tensor that is reduced every step (see :class:`BucketizedAllreduce`).
 
     Returns a work whose future completes with the tensor.  The result is in
     ``tensor`` once the work has been waited on, in stream order of the stream
@@ -137,7 +142,7 @@ def allreduce(
         divide_by = num_participants if reduce_op == ReduceOp.AVG and fold_normalization else None
         normalized = divide_by is not None
         work = allreduce_quantized([tensor], pg_reduce_op, process_group, torch.cuda.current_stream(),
-                                   divide_by=divide_by)
+                                   divide_by=divide_by, prepared=prepared)
     else:
         opts = AllreduceOptions()
         opts.reduceOp = pg_reduce_op
@@ -195,6 +200,90 @@ def _copy_all(dst: list, src: list) -> None:
             d.copy_(s)
 
 
+class BucketizedAllreduce:
+    """DiLoCo's bucket packing (local_sgd.py:499-556) with everything that does not change
+    from step to step built once: the flat buffers, the views of the tensors inside them and,
+    on the quantized path, one prepared bucket per flat buffer, so that a step costs the
+    copies and a few microseconds of host time per bucket.
+
+    The packing is the reference's (:func:`plan_buckets`), including its corner: tensors that
+    end up in no buffer keep their local values.  A bucket capacity that is a multiple of
+    every tensor's size, or larger than the whole list, avoids it.
+
+    One instance serves one list of tensors; steps on the same instance must not overlap
+    (wait for the works of a step before starting the next one: they share the flat buffers).
+    """
+
+    def __init__(self, tensors: list, bucket_size_bytes: int, row_width: int | None = None) -> None:
+        self.tensors = list(tensors)
+        self.row_width = row_width
+        self.buckets: list = []
+        if not self.tensors:
+            return
+        first = self.tensors[0]
+        capacity = bucket_size_bytes // first.element_size()
+        assert capacity > 0, "bucket_size_bytes is smaller than one element"
+        for length, members in plan_buckets([t.numel() for t in self.tensors], capacity):
+            padded = length
+            if row_width:
+                padded = -(-length // row_width) * row_width  # whole rows; the tail stays zero
+            flat = torch.zeros(padded, dtype=first.dtype, device=first.device)  # zero-filled (:527-529)
+            owners, pieces, at = [], [], 0
+            for i in members:
+                n = self.tensors[i].numel()
+                owners.append(self.tensors[i])
+                pieces.append(flat[at:at + n].view_as(self.tensors[i]))
+                at += n
+            self.buckets.append({"flat": flat, "view": flat.view(-1, row_width) if row_width else flat,
+                                 "owners": owners, "pieces": pieces, "used": at, "prepared": {}, "fresh": True})
+
+    def _pack(self, bucket: dict) -> None:
+        if not bucket["fresh"] and bucket["used"] < bucket["flat"].numel():
+            bucket["flat"][bucket["used"]:].zero_()  # what no tensor covers is zero in every step (:527-529)
+        bucket["fresh"] = False
+        _copy_all(bucket["pieces"], bucket["owners"])  # :534-537
+
+    @staticmethod
+    def _unpack_later(work: Any, bucket: dict) -> None:
+        owners, pieces = bucket["owners"], bucket["pieces"]
+
+        def unpack(fut):
+            _copy_all(owners, pieces)  # :546-551
+            return []
+
+        work.get_future().then(unpack)
+
+    def __call__(self, allreduce_fn: Callable[[torch.Tensor], Any]) -> list:
+        """Packs, calls ``allreduce_fn(flat)`` for every bucket and returns the works; each
+        tensor holds its reduced values once its bucket's work has been waited on."""
+        works = []
+        for bucket in self.buckets:
+            self._pack(bucket)
+            work = allreduce_fn(bucket["view"])
+            self._unpack_later(work, bucket)
+            works.append(work)
+        return works
+
+    def allreduce(self, process_group: Any, num_participants: int, is_participating: bool = True,
+                  should_quantize: bool = True, reduce_op: ReduceOp = ReduceOp.AVG) -> list:
+        """One managed all-reduce (:func:`allreduce`) per bucket; the quantized path reuses the
+        buckets' prepared tensor lists."""
+        works = []
+        ws = process_group.size()
+        for bucket in self.buckets:
+            self._pack(bucket)
+            prepared = None
+            if should_quantize:
+                prepared = bucket["prepared"].get(ws)
+                if prepared is None:
+                    prepared = bucket["prepared"][ws] = _q.prepare([bucket["view"]], ws)
+            work = allreduce(bucket["view"], process_group, num_participants, is_participating,
+                             should_quantize, reduce_op, prepared=prepared)
+            self._unpack_later(work, bucket)
+            works.append(work)
+        return works
+
+
 def bucketize_and_allreduce(
     tensors: list,
     bucket_size_bytes: int,
@@ -204,41 +293,11 @@ def bucketize_and_allreduce(
     """
     All-reduce ``tensors`` through flat buffers of at most ``bucket_size_bytes``
     (local_sgd.py:499-556) and return the works; each tensor holds its reduced
-    values once its bucket's work has been waited on.
-
-    The packing is the reference's (:func:`plan_buckets`), including its corner: tensors
-    that end up in no buffer keep their local values.  A bucket capacity that is a multiple
-    of every tensor's size, or larger than the whole list, avoids it.
+    values once its bucket's work has been waited on.  The flat buffers are allocated
+    for this call, as in the reference; :class:`BucketizedAllreduce` keeps them from
+    step to step.
 
     ``allreduce_fn(flat)`` is, for example,
     ``lambda t: allreduce(t, pg, n, should_quantize=True)``.
     """
-    if not tensors:
-        return []
-    first = tensors[0]
-    capacity = bucket_size_bytes // first.element_size()
-    assert capacity > 0, "bucket_size_bytes is smaller than one element"
-
-    works = []
-    for length, members in plan_buckets([t.numel() for t in tensors], capacity):
-        padded = length
-        if row_width:
-            padded = -(-length // row_width) * row_width  # whole rows; the tail stays zero
-        flat = torch.zeros(padded, dtype=first.dtype, device=first.device)  # zero-filled (:527-529)
-        owners, pieces, at = [], [], 0
-        for i in members:
-            n = tensors[i].numel()
-            owners.append(tensors[i])
-            pieces.append(flat[at:at + n].view_as(tensors[i]))
-            at += n
-        _copy_all(pieces, owners)  # :534-537
-
-        work = allreduce_fn(flat.view(-1, row_width) if row_width else flat)
-
-        def unpack(fut, owners=owners, pieces=pieces):
-            _copy_all(owners, pieces)  # :546-551
-            return []
-
-        work.get_future().then(unpack)
-        works.append(work)
-    return works
+    return BucketizedAllreduce(tensors, bucket_size_bytes, row_width)(allreduce_fn)

@@ -163,13 +163,14 @@ def reduce_scatter_quantized(
     ]
 
     with cuda.stream(ex.stream):
-        plan, device = _q._prepare(inputs, ws)  # one walk over the list for both kernels
-        packed = _q._quantize(plan, device)
+        bucket = _q.prepare(inputs, ws)  # one walk over the list for both kernels
+        packed = bucket.quantize()
         received, work = ex.scatter_slots(packed)
         work.wait()
 
         def reduce_then_dequantize() -> None:
-            _q._reduce(plan, device, received, rank, ex.reduce_op)
+            # `bucket` keeps the inputs alive, `share_views` the output, until this has been queued
+            bucket.reduce(received, rank, ex.reduce_op)
             own = received.view(ws, -1).split(1)[rank].squeeze(0)
             # one slot has the layout of a group of one over the [m_pad / ws, n] shares
             _q.fused_dequantize_from_fp8(share_views, own, 1)
@@ -185,6 +186,7 @@ def allreduce_quantized(
     sync_stream: cuda.Stream | None = None,
     *,
     divide_by: float | None = None,
+    prepared: "_q.PreparedBucket | None" = None,
 ):
     """
     Quantized all-reduce of ``tensors`` in place.  Only AVG and SUM are
@@ -196,18 +198,28 @@ def allreduce_quantized(
     left as if each had then been divided by that Python number on the GPU, as
     ``Manager.allreduce`` does with the number of participants
     (manager.py:450-452), at no extra pass over them.
+
+    ``prepared`` (no counterpart either): the result of
+    :func:`torchft_amd.quantization.prepare` for these very tensors and this group size.
+    A bucket that is reduced every step prepares once and passes it in, which takes the walk
+    over the tensor list out of every step.
     """
     ex = _begin(opts, AllreduceOptions, "allreduce", process_group, sync_stream)
     ws, rank = ex.world_size, ex.rank
 
+    if prepared is not None and (prepared.ws != ws or len(prepared.tensors) != len(tensors)):
+        raise ValueError("`prepared` was made for another tensor list or group size")
+
     with cuda.stream(ex.stream):
-        plan, device = _q._prepare(tensors, ws)  # one walk over the list for all three kernels
-        packed = _q._quantize(plan, device)
+        # one walk over the list for all three kernels; the bucket holds the tensors, so the
+        # memory behind the addresses it has bound outlives the dequantize kernel queued below
+        bucket = prepared if prepared is not None else _q.prepare(tensors, ws)
+        packed = bucket.quantize()
         received, a2a = ex.scatter_slots(packed)
         a2a.wait()
-        _q._reduce(plan, device, received, rank, ex.reduce_op)
+        bucket.reduce(received, rank, ex.reduce_op)
         # the reduced slots of all ranks land in the first buffer
         work = ex.gather_slots(packed, received)
         work.wait()  # a stream dependency with RCCL, not a host block
-        ex.finish_on_stream(work, lambda: _q._dequantize(plan, device, packed, divide_by))
+        ex.finish_on_stream(work, lambda: bucket.dequantize(packed, divide_by))
     return work

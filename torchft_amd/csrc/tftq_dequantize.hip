@@ -311,28 +311,25 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
 template <typename T, bool POST>
 static int launch_d(const KParams &kp, const InlineTable &inl, bool use_inline, hipStream_t st)
 {
-    if (use_inline)
-        hipLaunchKernelGGL((k_dequantize<T, true, POST>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
-    else
-        hipLaunchKernelGGL((k_dequantize<T, false, POST>), dim3(grid_of(kp)), dim3(TFTQ_WG), 0, st, kp, inl);
-    return (int)hipGetLastError();
+    if (use_inline) return launch_kernel(k_dequantize<T, true, POST>, grid_of(kp), 0, st, kp, inl);
+    return launch_kernel(k_dequantize<T, false, POST>, grid_of(kp), 0, st, kp, inl);
 }
 
 template <bool POST>
-static int dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes, float post_scale,
-                      void *stream)
+static int dequantize(const tftq_plan *plan, void *const *tensors, const void *table, void *pointers,
+                      const void *packed, int64_t packed_bytes, float post_scale, int device, void *stream)
 {
     KParams kp;
     InlineTable inl = {};
     bool use_inline;
-    int rc = fill_params(plan, ST_D, (void *)packed, packed_bytes, &kp, &inl, &use_inline);
+    hipStream_t st = (hipStream_t)stream;
+    DeviceScope scope(device);
+    if (scope.err != hipSuccess) return (int)scope.err;
+    int rc = fill_params(plan, ST_D, (const void *const *)tensors, table, pointers, (void *)packed, packed_bytes, st,
+                         &kp, &inl, &use_inline);
     if (rc) return rc;
     kp.post_scale = post_scale;
-    for (int i = 0; i < plan->nseg; i++)
-        if (plan->segs[(size_t)i].ptr == 0 && plan->segs[(size_t)i].m > 0 && plan->segs[(size_t)i].n > 0)
-            return TFTQ_E_ARG;
     if (kp.nwg == 0) return 0;
-    hipStream_t st = (hipStream_t)stream;
     switch (plan->dtype) {
     case TFTQ_F32: return launch_d<float, POST>(kp, inl, use_inline, st);
     case TFTQ_F16: return launch_d<f16_tag, POST>(kp, inl, use_inline, st);
@@ -341,14 +338,15 @@ static int dequantize(const tftq_plan *plan, const void *packed, int64_t packed_
     }
 }
 
-extern "C" int tftq_dequantize(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
-                               void *stream)
+extern "C" int tftq_dequantize(const tftq_plan *plan, void *const *tensors, const void *table, void *pointers,
+                               const void *packed, int64_t packed_bytes, int device, void *stream)
 {
-    return dequantize<false>(plan, packed, packed_bytes, 1.0f, stream);
+    return dequantize<false>(plan, tensors, table, pointers, packed, packed_bytes, 1.0f, device, stream);
 }
 
-extern "C" int tftq_dequantize_scaled(const tftq_plan *plan, const void *packed, int64_t packed_bytes,
-                                      float post_scale, void *stream)
+extern "C" int tftq_dequantize_scaled(const tftq_plan *plan, void *const *tensors, const void *table,
+                                      void *pointers, const void *packed, int64_t packed_bytes,
+                                      float post_scale, int device, void *stream)
 {
-    return dequantize<true>(plan, packed, packed_bytes, post_scale, stream);
+    return dequantize<true>(plan, tensors, table, pointers, packed, packed_bytes, post_scale, device, stream);
 }

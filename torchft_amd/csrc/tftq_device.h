@@ -380,8 +380,8 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
         return true;
     } else {
         // everything the first steps need from the kernel arguments in one round of scalar loads
-        asm volatile("" ::"s"(p.table), "s"(p.map_off), "s"(p.sorted_off), "s"(p.map_shift), "s"(p.chunk_shift), "s"(p.nwg),
-                     "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
+        asm volatile("" ::"s"(p.table), "s"(p.ptrs), "s"(p.map_off), "s"(p.sorted_off), "s"(p.map_shift), "s"(p.chunk_shift),
+                     "s"(p.nwg), "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
         // chunks of 2^chunk_shift consecutive workgroups go to the XCDs in turn
         const int cs = p.chunk_shift;
         vb = ((((i >> cs) << 3) + x) << cs) + (i & ((1 << cs) - 1));
@@ -401,7 +401,11 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
         }
         const CONSTANT u32x4 *src = (const CONSTANT u32x4 *)(tab + (uint64_t)sg * sizeof(Seg));
         const u32x4 v[4] = {src[0], src[1], src[2], src[3]};
+        // the table holds no addresses: the tensor's comes from the call's pointer array
+        uint64_t tptr = 0;
+        if (STAGE != ST_R) tptr = *(const CONSTANT uint64_t *)((uint64_t)p.ptrs + (uint64_t)sg * 8u);
         __builtin_memcpy(&s, v, sizeof(Seg));
+        s.ptr = tptr;
         return true;
     }
 }
@@ -464,8 +468,51 @@ static inline void work_mapping(const tftq_plan *plan, int stage, KParams *kp)
     }
 }
 
-static inline int fill_params(const tftq_plan *plan, int stage, void *packed, int64_t packed_bytes,
-                       KParams *kp, InlineTable *inl, bool *use_inline)
+// Makes `device` current for the lifetime of the object and restores the caller's device
+// afterwards; device < 0 leaves the current device alone.
+struct DeviceScope {
+    int prev = -1;
+    bool switched = false;
+    hipError_t err = hipSuccess;
+    explicit DeviceScope(int device)
+    {
+        if (device < 0) return;
+        err = hipGetDevice(&prev);
+        if (err == hipSuccess && prev != device) {
+            err = hipSetDevice(device);
+            switched = err == hipSuccess;
+        }
+    }
+    ~DeviceScope()
+    {
+        if (switched) (void)hipSetDevice(prev);
+    }
+    DeviceScope(const DeviceScope &) = delete;
+    DeviceScope &operator=(const DeviceScope &) = delete;
+};
+
+// Copies `bytes` bytes (a multiple of 8) from host memory to 8-byte aligned device memory
+// with small kernels on `st` that carry the data in their arguments: the source is read
+// before the function returns, nothing is allocated or synchronised, and a stream capture
+// records the data itself.  Defined in tftq_runtime.hip.
+__attribute__((visibility("hidden"))) int tftq_put_bytes(void *dst_device, const void *src_host, size_t bytes,
+                                                         hipStream_t st);
+
+// One kernel launch with the launch's own error (not whatever an earlier call left behind).
+template <typename K>
+static inline int launch_kernel(K kernel, unsigned grid, unsigned lds_bytes, hipStream_t st, const KParams &kp,
+                                const InlineTable &inl)
+{
+    void *args[2] = {(void *)&kp, (void *)&inl};
+    return (int)hipLaunchKernel((const void *)kernel, dim3(grid), dim3(TFTQ_WG), args, lds_bytes, st);
+}
+
+// Kernel parameters of one call.  tensors: host array of the tensors' device addresses (null
+// in reduce); table / pointers: the caller's device buffers of a long list.  For a long list
+// with `tensors` the addresses are written to `pointers` on `st` first.
+static inline int fill_params(const tftq_plan *plan, int stage, const void *const *tensors, const void *table,
+                              void *pointers, void *packed, int64_t packed_bytes, hipStream_t st, KParams *kp,
+                              InlineTable *inl, bool *use_inline)
 {
     if (!plan) return TFTQ_E_ARG;
     if (packed_bytes != plan->output_size) return TFTQ_E_SIZE;
@@ -473,8 +520,30 @@ static inline int fill_params(const tftq_plan *plan, int stage, void *packed, in
     if (!packed && plan->output_size != 0) return TFTQ_E_ARG;
     if (((uintptr_t)packed & 3) != 0) return TFTQ_E_ARG;
     *use_inline = plan->nseg <= TFTQ_N_INLINE;
-    if (!*use_inline && !plan->device_table) return TFTQ_E_NOTABLE;
-    kp->table = *use_inline ? nullptr : (const Seg *)plan->device_table;
+    const bool needs_tensors = stage != ST_R && plan->nwg[stage] > 0;
+    if (*use_inline) {
+        if (needs_tensors && !tensors) return TFTQ_E_ARG;
+        for (int i = 0; i < plan->nseg; i++) {
+            inl->s[i] = plan->segs[(size_t)i];
+            if (stage != ST_R) {
+                inl->s[i].ptr = (uint64_t)(uintptr_t)(tensors ? tensors[i] : nullptr);
+                if (inl->s[i].ptr == 0 && inl->s[i].m > 0 && inl->s[i].n > 0) return TFTQ_E_ARG;
+            }
+        }
+    } else if (plan->nwg[stage] > 0) {
+        if (!table || ((uintptr_t)table & 255) != 0) return TFTQ_E_NOTABLE;
+        if (needs_tensors) {
+            if (!pointers || ((uintptr_t)pointers & 7) != 0) return TFTQ_E_NOTABLE;
+            if (tensors) {
+                for (int i = 0; i < plan->nseg; i++)
+                    if (!tensors[i] && plan->segs[(size_t)i].m > 0 && plan->segs[(size_t)i].n > 0) return TFTQ_E_ARG;
+                const int rc = tftq_put_bytes(pointers, tensors, (size_t)plan->nseg * 8, st);
+                if (rc) return rc;
+            }
+        }
+    }
+    kp->table = *use_inline ? nullptr : (const Seg *)table;
+    kp->ptrs = (*use_inline || stage == ST_R) ? nullptr : (const uint64_t *)pointers;
     kp->packed = (uint8_t *)packed;
     kp->slot_size = plan->slot_size;
     kp->nseg = plan->nseg;
@@ -486,8 +555,6 @@ static inline int fill_params(const tftq_plan *plan, int stage, void *packed, in
     kp->div = 1.0f;
     kp->inv_div = 1.0f;
     kp->post_scale = 1.0f;
-    if (*use_inline)
-        for (int i = 0; i < plan->nseg; i++) inl->s[i] = plan->segs[(size_t)i];
     return 0;
 }
 

@@ -6,6 +6,8 @@
 
 #include <vector>
 
+#include "../../include/tftq.h"
+
 // Stages of the path, used to index per-stage fields of a segment.
 enum : int { ST_Q = 0, ST_R = 1, ST_D = 2 };
 
@@ -101,7 +103,7 @@ TFTQ_HD static inline int tftq_col1_rows_per_wg(int stage)
                          : 4 * TFTQ_WG;
 }
 
-constexpr int TFTQ_N_INLINE = 16;  // segments that travel in the kernel arguments
+// TFTQ_N_INLINE (tftq.h): segments that travel in the kernel arguments
 
 // Rows a workgroup can hold in registers.  The regular kernels keep up to 8
 // input vectors per lane in quantize (rows of 2048 vectors = 32 KB) and the
@@ -117,7 +119,7 @@ constexpr int TFTQ_R_DWORDS = 4096, TFTQ_R_DWORDS_WIDE = 8192;
 
 // One tensor of the list.  64 bytes.
 struct Seg {
-    uint64_t ptr;        // device address of element (0,0); 0 for reduce-only plans
+    uint64_t ptr;        // device address of element (0,0): 0 in the plan and in the table image, set per call
     int64_t slot_off;    // byte offset of this tensor's rows inside every slot
     int64_t row_stride;  // elements
     int64_t col_stride;  // elements
@@ -194,12 +196,12 @@ struct tftq_plan {
     TableIndex index[3];       // device table only
     std::vector<Seg> segs;
     std::vector<uint8_t> blob;  // host image of the device table (nseg > TFTQ_N_INLINE)
-    const void *device_table;   // set by the caller when nseg > TFTQ_N_INLINE
 };
 
 // Kernel parameters common to the three stages.
 struct KParams {
     const Seg *table;   // device table, or nullptr when the inline table is used
+    const uint64_t *ptrs;  // device table only: the tensors' addresses, in list order (null in reduce)
     uint8_t *packed;
     int64_t slot_size;
     int32_t nseg;

@@ -20,6 +20,11 @@ static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 extern "C" int tftq_version(void) { return TFTQ_VERSION; }
 
+#ifndef TFTQ_BUILD_ID
+#define TFTQ_BUILD_ID "unknown"
+#endif
+extern "C" const char *tftq_build_id(void) { return TFTQ_BUILD_ID; }
+
 extern "C" const char *tftq_strerror(int code)
 {
     switch (code) {
@@ -29,7 +34,7 @@ extern "C" const char *tftq_strerror(int code)
     case TFTQ_E_SHAPE: return "tensor dimension out of range";
     case TFTQ_E_SIZE: return "Output size does not match";
     case TFTQ_E_NOMEM: return "out of host memory";
-    case TFTQ_E_NOTABLE: return "plan needs a device descriptor table";
+    case TFTQ_E_NOTABLE: return "a list of more than 16 tensors needs the device table and the pointer buffer";
     case TFTQ_E_ARCH: return "device is not gfx950";
     default: return code > 0 ? "HIP error" : "unknown error";
     }
@@ -59,10 +64,10 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     // row length needs to be a multiple of 16 bytes: gfx950 loads and stores 16-byte
     // vectors at element alignment, and a short tail is handled per element.
     const int64_t in_bytes = (int64_t)s.n * esz;
-    const bool vec_ok = s.ptr != 0 && s.col_stride == 1 && in_bytes >= 64;
-    if (s.n == 1 && s.ptr != 0) return K_COL1;
+    const bool vec_ok = s.col_stride == 1 && in_bytes >= 64;
+    if (s.n == 1) return K_COL1;
     const int epv = 16 / esz;
-    if (s.ptr != 0 && s.col_stride == 1 && s.n % epv == 0 && s.n / epv >= 1 && s.n / epv <= 32)
+    if (s.col_stride == 1 && s.n % epv == 0 && s.n / epv >= 1 && s.n / epv <= 32)
         return K_VECS;  // short rows of whole vectors
     if (vec_ok) {
         // Team sizes measured on MI355X inside quantize -> reduce -> dequantize sequences (a
@@ -242,9 +247,8 @@ static int build_table(tftq_plan *p, const int32_t (*wgs)[3])
     return 0;
 }
 
-extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptrs,
-                                const int64_t *shapes, const int64_t *strides, int ws,
-                                tftq_plan **out)
+extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes, const int64_t *strides,
+                                int ws, tftq_plan **out)
 {
     if (!out) return TFTQ_E_ARG;
     *out = nullptr;
@@ -257,33 +261,28 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const void *const *ptr
     p->esz = dtype == TFTQ_F32 ? 4 : 2;
     p->ws = ws;
     p->nseg = n_tensors;
-    p->device_table = nullptr;
     p->max_rows = 0;
-    try {
+    std::vector<int64_t> offs;
+    std::vector<int32_t> wgs_flat;
+    try {  // nothing may throw across the C ABI
         p->segs.resize((size_t)n_tensors);
+        offs.resize((size_t)n_tensors);
+        wgs_flat.resize((size_t)n_tensors * 3);
     } catch (...) {
         delete p;
         return TFTQ_E_NOMEM;
     }
-    std::vector<int64_t> offs((size_t)n_tensors);
     int rc = tftq_layout(n_tensors, shapes, ws, offs.data(), &p->slot_size, &p->output_size);
     if (rc) {
         delete p;
         return rc;
     }
     int64_t wg[3] = {0, 0, 0};
-    std::vector<int32_t> wgs_flat;
-    try {
-        wgs_flat.resize((size_t)n_tensors * 3);
-    } catch (...) {
-        delete p;
-        return TFTQ_E_NOMEM;
-    }
     int32_t (*wgs)[3] = (int32_t (*)[3])wgs_flat.data();  // workgroups per segment and stage
     for (int i = 0; i < n_tensors; i++) {
         Seg &s = p->segs[(size_t)i];
         memset(&s, 0, sizeof(s));
-        s.ptr = ptrs ? (uint64_t)(uintptr_t)ptrs[i] : 0;
+        s.ptr = 0;
         s.slot_off = offs[(size_t)i];
         s.m = (int32_t)shapes[2 * i];
         s.n = (int32_t)shapes[2 * i + 1];
@@ -343,6 +342,7 @@ extern "C" void tftq_plan_destroy(tftq_plan *plan) { delete plan; }
 extern "C" int64_t tftq_plan_output_size(const tftq_plan *plan) { return plan ? plan->output_size : -1; }
 extern "C" int64_t tftq_plan_slot_size(const tftq_plan *plan) { return plan ? plan->slot_size : -1; }
 extern "C" int64_t tftq_plan_max_rows(const tftq_plan *plan) { return plan ? plan->max_rows : -1; }
+extern "C" int tftq_plan_n_tensors(const tftq_plan *plan) { return plan ? plan->nseg : -1; }
 
 extern "C" int64_t tftq_plan_table_bytes(const tftq_plan *plan)
 {
@@ -353,12 +353,5 @@ extern "C" int64_t tftq_plan_table_bytes(const tftq_plan *plan)
 extern "C" const void *tftq_plan_table_host(const tftq_plan *plan)
 {
     if (!plan) return nullptr;
-    return plan->nseg > TFTQ_N_INLINE ? (const void *)plan->blob.data() : (const void *)plan->segs.data();
-}
-
-extern "C" int tftq_plan_set_device_table(tftq_plan *plan, const void *device_table)
-{
-    if (!plan) return TFTQ_E_ARG;
-    plan->device_table = device_table;
-    return 0;
+    return plan->nseg > TFTQ_N_INLINE ? (const void *)plan->blob.data() : nullptr;
 }

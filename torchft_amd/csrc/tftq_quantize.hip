@@ -423,30 +423,28 @@ template <typename T>
 static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, bool parked,
                     hipStream_t st)
 {
-    const dim3 grid(grid_of(kp)), block(TFTQ_WG);
+    const unsigned grid = grid_of(kp);
     if (wide) {
         const unsigned lds = parked ? TFTQ_Q_PARKED * TFTQ_WG * 16u : 0u;
-        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, true>), grid, block, lds, st, kp, inl);
-        else hipLaunchKernelGGL((k_quantize<T, false, true>), grid, block, lds, st, kp, inl);
-    } else {
-        if (use_inline) hipLaunchKernelGGL((k_quantize<T, true, false>), grid, block, 0, st, kp, inl);
-        else hipLaunchKernelGGL((k_quantize<T, false, false>), grid, block, 0, st, kp, inl);
+        if (use_inline) return launch_kernel(k_quantize<T, true, true>, grid, lds, st, kp, inl);
+        return launch_kernel(k_quantize<T, false, true>, grid, lds, st, kp, inl);
     }
-    return (int)hipGetLastError();
+    if (use_inline) return launch_kernel(k_quantize<T, true, false>, grid, 0, st, kp, inl);
+    return launch_kernel(k_quantize<T, false, false>, grid, 0, st, kp, inl);
 }
 
-extern "C" int tftq_quantize(const tftq_plan *plan, void *packed, int64_t packed_bytes, void *stream)
+extern "C" int tftq_quantize(const tftq_plan *plan, const void *const *tensors, const void *table,
+                             void *pointers, void *packed, int64_t packed_bytes, int device, void *stream)
 {
     KParams kp;
     InlineTable inl = {};
     bool use_inline;
-    int rc = fill_params(plan, ST_Q, packed, packed_bytes, &kp, &inl, &use_inline);
-    if (rc) return rc;
-    for (int i = 0; i < plan->nseg; i++)
-        if (plan->segs[(size_t)i].ptr == 0 && plan->segs[(size_t)i].m > 0 && plan->segs[(size_t)i].n > 0)
-            return TFTQ_E_ARG;
-    if (kp.nwg == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
+    DeviceScope scope(device);
+    if (scope.err != hipSuccess) return (int)scope.err;
+    int rc = fill_params(plan, ST_Q, tensors, table, pointers, packed, packed_bytes, st, &kp, &inl, &use_inline);
+    if (rc) return rc;
+    if (kp.nwg == 0) return 0;
     switch (plan->dtype) {
     case TFTQ_F32: return launch_q<float>(kp, inl, use_inline, plan->wide[ST_Q], plan->parked, st);
     case TFTQ_F16: return launch_q<f16_tag>(kp, inl, use_inline, plan->wide[ST_Q], plan->parked, st);

@@ -878,27 +878,14 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
 // ---------------------------------------------------------------------------
 // C ABI
 // ---------------------------------------------------------------------------
-extern "C" int tftq_check_device(void)
-{
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    hipDeviceProp_t prop;
-    e = hipGetDeviceProperties(&prop, dev);
-    if (e != hipSuccess) return (int)e;
-    const char *a = prop.gcnArchName;
-    return (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')
-               ? 0
-               : TFTQ_E_ARCH;
-}
-
-extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank,
-                           int is_avg, void *stream)
+// The launch of tftq_reduce with the device already current.
+static int reduce_launch(const tftq_plan *plan, const void *table, void *packed, int64_t packed_bytes, int rank,
+                         int is_avg, hipStream_t st)
 {
     KParams kp;
     InlineTable inl = {};
     bool use_inline;
-    int rc = fill_params(plan, ST_R, packed, packed_bytes, &kp, &inl, &use_inline);
+    int rc = fill_params(plan, ST_R, nullptr, table, nullptr, packed, packed_bytes, st, &kp, &inl, &use_inline);
     if (rc) return rc;
     if (rank < 0 || rank >= plan->ws) return TFTQ_E_ARG;
     kp.rank = rank;
@@ -916,10 +903,9 @@ extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_b
         }
     }
     if (kp.nwg == 0) return 0;
-    hipStream_t st = (hipStream_t)stream;
-    const dim3 grid(grid_of(kp)), block(TFTQ_WG);
+    const unsigned grid = grid_of(kp);
     const bool gdiv = kp.div_mode >= 2;
-#define TFTQ_LAUNCH_R(I, G, W) hipLaunchKernelGGL((k_reduce<I, G, W>), grid, block, 0, st, kp, inl)
+#define TFTQ_LAUNCH_R(I, G, W) return launch_kernel(k_reduce<I, G, W>, grid, 0, st, kp, inl)
     if (plan->wide[ST_R]) {
         if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, true); else TFTQ_LAUNCH_R(false, true, true); }
         else { if (use_inline) TFTQ_LAUNCH_R(true, false, true); else TFTQ_LAUNCH_R(false, false, true); }
@@ -928,5 +914,12 @@ extern "C" int tftq_reduce(const tftq_plan *plan, void *packed, int64_t packed_b
         else { if (use_inline) TFTQ_LAUNCH_R(true, false, false); else TFTQ_LAUNCH_R(false, false, false); }
     }
 #undef TFTQ_LAUNCH_R
-    return (int)hipGetLastError();
+}
+
+extern "C" int tftq_reduce(const tftq_plan *plan, const void *table, void *packed, int64_t packed_bytes, int rank,
+                           int is_avg, int device, void *stream)
+{
+    DeviceScope scope(device);
+    if (scope.err != hipSuccess) return (int)scope.err;
+    return reduce_launch(plan, table, packed, packed_bytes, rank, is_avg, (hipStream_t)stream);
 }

@@ -12,8 +12,16 @@ observe:
   by the quantize kernel, instead of ``torch.zeros`` plus a kernel
   (quantization.py:567-571); the bytes are identical;
 * the per-call host work of ``_prepare_quantize_fp8`` (four device tables and
-  five allocations per call, quantization.py:505-517) is replaced by a cached
-  plan; lists of up to 16 tensors need no device metadata at all.
+  five allocations per call, quantization.py:505-517) is replaced by a plan that
+  depends on shapes, strides, dtype and group size only and is cached; the
+  tensors' addresses travel with each call.  Lists of up to 16 tensors need no
+  device metadata at all; longer lists use one cached descriptor table per
+  device and 8 bytes per tensor for the addresses.
+
+:func:`prepare` (no counterpart in the reference) does the walk over a tensor
+list once and returns a :class:`PreparedBucket` whose ``quantize`` / ``reduce`` /
+``dequantize`` cost the same few microseconds whatever the length of the list:
+the thing to hold on to for a bucket that is reduced every step.
 
 There is no CPU or eager fallback: without the HIP library and a gfx950 device
 the functions raise.
@@ -39,26 +47,73 @@ SCALE_DTYPE_BYTES: int = 4
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 _TENSOR = torch.Tensor
 _DTYPE_OF = operator.attrgetter("dtype")
-# Plans are cached by (device, dtype, group size, addresses, shapes, strides).  The
-# per-parameter all-reduce of a model has one single-tensor plan per parameter, so the
-# cache holds thousands of small plans; long lists are bounded by their total length.
+_N_INLINE = 16  # TFTQ_N_INLINE
+# Plans are cached by (dtype, group size, shapes, strides).  The per-parameter all-reduce of a
+# model has one single-tensor plan per distinct shape; long lists are bounded by their total
+# length.
 _PLAN_CACHE_SIZE = 4096
 _PLAN_CACHE_TENSORS = 1 << 18
 
 
+class _Ready:
+    """An upload that kernels on other streams must wait for until it has completed."""
+
+    __slots__ = ("event", "stream_id")
+
+    def __init__(self, stream: torch.cuda.Stream) -> None:
+        self.event: torch.cuda.Event | None = torch.cuda.Event()
+        self.event.record(stream)
+        self.stream_id = stream.cuda_stream
+
+    def wait(self, stream: torch.cuda.Stream, raw_stream: int) -> None:
+        ev = self.event
+        if ev is None or raw_stream == self.stream_id:  # done, or ordered by the stream itself
+            return
+        if ev.query():
+            self.event = None
+        else:
+            stream.wait_event(ev)
+
+
 class _Plan:
-    """Owns a ``tftq_plan`` and, for long tensor lists, its device table."""
+    """Owns a ``tftq_plan`` and, for long tensor lists, its descriptor table on every
+    device it has been used on.  Holds no tensor and no address."""
 
-    __slots__ = ("handle", "output_size", "slot_size", "max_rows", "table", "n_tensors", "_lib")
+    __slots__ = ("handle", "output_size", "slot_size", "max_rows", "n_tensors", "table_bytes",
+                 "tables", "_lib", "_lock")
 
-    def __init__(self, lib, handle, table, n_tensors):
+    def __init__(self, lib, handle, n_tensors):
         self._lib = lib
         self.handle = handle
-        self.table = table
         self.n_tensors = n_tensors
         self.output_size = lib.tftq_plan_output_size(handle)
         self.slot_size = lib.tftq_plan_slot_size(handle)
         self.max_rows = lib.tftq_plan_max_rows(handle)
+        self.table_bytes = lib.tftq_plan_table_bytes(handle)
+        self.tables: dict = {}  # device index -> (device tensor, _Ready)
+        self._lock = threading.Lock()
+
+    def table_on(self, device: torch.device):
+        """The descriptor table on ``device`` (None for short lists).  The first use on a
+        device copies the image from pinned staging memory on the current stream; nothing
+        blocks, and users on other streams wait for the copy's event."""
+        if self.table_bytes == 0:
+            return None
+        entry = self.tables.get(device.index)
+        if entry is None:
+            with self._lock:
+                entry = self.tables.get(device.index)
+                if entry is None:
+                    host = (ctypes.c_uint8 * self.table_bytes).from_address(
+                        self._lib.tftq_plan_table_host(self.handle))
+                    staged = torch.empty(self.table_bytes, dtype=torch.uint8, pin_memory=True)
+                    staged.copy_(torch.frombuffer(host, dtype=torch.uint8))
+                    with torch.cuda.device(device):
+                        table = torch.empty(self.table_bytes, dtype=torch.uint8, device=device)
+                        table.copy_(staged, non_blocking=True)  # the pinned allocator keeps `staged` until then
+                        entry = (table, _Ready(torch.cuda.current_stream(device)))
+                    self.tables[device.index] = entry
+        return entry
 
     def __del__(self):
         try:
@@ -104,52 +159,23 @@ def _validate(inputs: list[torch.Tensor]) -> tuple[torch.device, torch.dtype]:
     return device, dtype
 
 
-def _prepare(inputs: list[torch.Tensor], all_reduce_group_size: int) -> tuple[_Plan, torch.device]:
-    """Counterpart of ``_prepare_quantize_fp8`` (quantization.py:431-528)."""
-    device, dtype = _validate(inputs)
-    if device.type != "cuda":
-        raise RuntimeError(
-            "torchft_amd.quantization needs tensors on a gfx950 GPU; there is no CPU path")
-    ws = int(all_reduce_group_size)
-    # The key holds tens of thousands of small tuples for long lists; keep the cyclic
-    # garbage collector from walking them while they are being built.
-    pause_gc = len(inputs) > 256 and gc.isenabled()
-    if pause_gc:
-        gc.disable()
-    try:
-        ptrs_key = tuple(map(_TENSOR.data_ptr, inputs))
-        sizes_key = tuple(map(_TENSOR.size, inputs))
-        strides_key = tuple(map(_TENSOR.stride, inputs))
-        key = (device.index, dtype, ws, ptrs_key, sizes_key, strides_key)
-    finally:
-        if pause_gc:
-            gc.enable()
+def _plan_for(dtype: torch.dtype, ws: int, sizes_key: tuple, strides_key: tuple) -> _Plan:
+    key = (dtype, ws, sizes_key, strides_key)
     with _cache_lock:
         plan = _plan_cache.get(key)
         if plan is not None:
             _plan_cache.move_to_end(key)
-            return plan, device
-
+            return plan
     lib = _lib.load()
-    T = len(inputs)
-    ptrs = (ctypes.c_void_p * T)()
+    T = len(sizes_key)
     shapes = (ctypes.c_int64 * (2 * T))()
     strides = (ctypes.c_int64 * (2 * T))()
-    ptrs[:] = ptrs_key
     shapes[:] = [d for sz in sizes_key for d in sz]
     strides[:] = [d for st in strides_key for d in st]
     handle = ctypes.c_void_p()
-    _check(lib.tftq_plan_create(_DTYPE_CODE[dtype], T, ptrs, shapes, strides, ws,
-                                ctypes.byref(handle)), "tftq_plan_create")
-    table = None
-    nbytes = lib.tftq_plan_table_bytes(handle)
-    if nbytes > 0:
-        host = (ctypes.c_uint8 * nbytes).from_address(lib.tftq_plan_table_host(handle))
-        # synchronous copy: the plan may be used from any stream afterwards
-        table = torch.frombuffer(host, dtype=torch.uint8).to(device)
-        _check(lib.tftq_plan_set_device_table(handle, ctypes.c_void_p(table.data_ptr())),
-               "tftq_plan_set_device_table")
-    plan = _Plan(lib, handle, table, T)
+    _check(lib.tftq_plan_create(_DTYPE_CODE[dtype], T, shapes, strides, ws, ctypes.byref(handle)),
+           "tftq_plan_create")
+    plan = _Plan(lib, handle, T)
     global _plan_cache_tensors
     with _cache_lock:
         old = _plan_cache.pop(key, None)  # another thread may have built the same plan
@@ -161,46 +187,144 @@ def _prepare(inputs: list[torch.Tensor], all_reduce_group_size: int) -> tuple[_P
                                         or _plan_cache_tensors > _PLAN_CACHE_TENSORS):
             _, gone = _plan_cache.popitem(last=False)
             _plan_cache_tensors -= gone.n_tensors
-    return plan, device
+    return plan
 
 
 # Per-call host cost matters for the per-parameter all-reduce (thousands of small
-# calls): the raw current stream and the current device come from torch's C
-# bindings where they exist (0.3 us instead of 4 us for a Stream object and
-# 2 us for a device context that changes nothing).
+# calls): the raw current stream comes from torch's C bindings where they exist
+# (0.3 us instead of 4 us for a Stream object).
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
-_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-def _stream_ptr(device: torch.device) -> ctypes.c_void_p:
-    if _raw_stream is not None and device.index is not None:
-        return ctypes.c_void_p(_raw_stream(device.index))
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+def _stream_of(device: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
-class _NoSwitch:
-    def __enter__(self):
-        return None
+class PreparedBucket:
+    """One list of tensors, ready for the three kernels: the result of :func:`prepare`.
 
-    def __exit__(self, *exc):
-        return False
+    Holds the plan, the tensors (so that their memory outlives every kernel queued on
+    their addresses) and, for lists of more than 16 tensors, the device copy of their
+    addresses.  The methods launch on the current stream of the tensors' device and cost
+    a few microseconds of host time whatever the length of the list.
 
+    The bucket is bound to the storage the tensors had when it was prepared: prepare again
+    after ``tensor.data = ...``, ``resize_`` or anything else that moves a tensor.  One
+    bucket may be used from several threads and streams.  A HIP graph that captures these
+    calls must be kept together with the bucket: it pins the plan's table and the
+    addresses that the captured kernels read.
+    """
 
-_NO_SWITCH = _NoSwitch()
+    __slots__ = ("plan", "device", "tensors", "ws", "_ptrs", "_ptrs_dev", "_ptrs_ready", "_table",
+                 "_table_ready", "_lib", "_handle", "_dev_index", "_lock")
 
+    def __init__(self, plan: _Plan, device: torch.device, tensors: list, ws: int, ptrs) -> None:
+        self.plan = plan
+        self.device = device
+        self.tensors = tensors
+        self.ws = ws
+        self._lib = plan._lib
+        self._handle = plan.handle
+        self._dev_index = device.index
+        self._ptrs = ptrs                # host array of addresses (ctypes)
+        self._ptrs_dev = None            # long lists: their device copy, written by the first call
+        self._ptrs_ready: _Ready | None = None
+        self._table = None
+        self._table_ready: _Ready | None = None
+        self._lock = threading.Lock()
+        if plan.table_bytes:
+            table, ready = plan.table_on(device)
+            self._table = table
+            self._table_ready = ready
+            with torch.cuda.device(device):
+                self._ptrs_dev = torch.empty(plan.n_tensors, dtype=torch.int64, device=device)
 
-def _on_device(device: torch.device):
-    """Context in which ``device`` is the current device."""
-    if _raw_device is not None and device.index is not None and _raw_device() == device.index:
-        return _NO_SWITCH
-    return torch.cuda.device(device)
+    # -- properties of the layout ------------------------------------------------------
+    @property
+    def output_size(self) -> int:
+        """Bytes of the packed buffer (``numel()`` of what :meth:`quantize` returns)."""
+        return self.plan.output_size
 
+    @property
+    def slot_size(self) -> int:
+        return self.plan.slot_size
 
-def _keep_table(plan: _Plan, device: torch.device) -> None:
-    """A plan can be evicted from the cache while its kernel is still queued: tell the
-    allocator on which stream the device table is in use."""
-    if plan.table is not None:
-        plan.table.record_stream(torch.cuda.current_stream(device))
+    # -- launches ------------------------------------------------------------------------
+    def _long_list_args(self, raw_stream: int, needs_pointers: bool):
+        """(table, pointers) arguments of a compute call on a long list, both current for
+        kernels on the current stream, and protected against being freed while in use there."""
+        stream = torch.cuda.current_stream(self.device)
+        self._table_ready.wait(stream, raw_stream)
+        self._table.record_stream(stream)
+        if not needs_pointers:
+            return self._table.data_ptr(), None
+        self._ptrs_dev.record_stream(stream)
+        ready = self._ptrs_ready
+        if ready is None:
+            with self._lock:
+                ready = self._ptrs_ready
+                if ready is None:
+                    # the first call on this bucket writes the addresses; later calls reuse them
+                    _check(self._lib.tftq_upload_pointers(self._handle, self._ptrs, self._ptrs_dev.data_ptr(),
+                                                          self._dev_index, raw_stream), "tftq_upload_pointers")
+                    self._ptrs_ready = _Ready(stream)
+                    return self._table.data_ptr(), self._ptrs_dev.data_ptr()
+        ready.wait(stream, raw_stream)
+        return self._table.data_ptr(), self._ptrs_dev.data_ptr()
+
+    def quantize(self, out: torch.Tensor | None = None) -> torch.Tensor:
+        """Quantizes the tensors into ``out`` (allocated when None) and returns it."""
+        plan = self.plan
+        if out is None:
+            out = torch.empty(plan.output_size, dtype=torch.uint8, device=self.device)
+        else:
+            _check_packed(out, plan, self.device)
+        raw = _stream_of(self.device)
+        if self._table is None:
+            rc = self._lib.tftq_quantize(self._handle, self._ptrs, None, None, out.data_ptr(),
+                                         plan.output_size, self._dev_index, raw)
+        else:
+            table, pointers = self._long_list_args(raw, True)
+            rc = self._lib.tftq_quantize(self._handle, None, table, pointers, out.data_ptr(),
+                                         plan.output_size, self._dev_index, raw)
+        _check(rc, "tftq_quantize")
+        return out
+
+    def reduce(self, packed: torch.Tensor, rank: int, reduce_op: ReduceOp = ReduceOp.SUM) -> None:
+        """Reduces the ``ws`` slots of ``packed`` into slot ``rank`` in place."""
+        plan = self.plan
+        _check_packed(packed, plan, self.device)
+        is_avg = 0 if reduce_op == ReduceOp.SUM else 1  # anything but SUM averages (:682)
+        raw = _stream_of(self.device)
+        table = None
+        if self._table is not None:
+            table, _ = self._long_list_args(raw, False)
+        _check(self._lib.tftq_reduce(self._handle, table, packed.data_ptr(), plan.output_size, int(rank), is_avg,
+                                     self._dev_index, raw), "tftq_reduce")
+
+    def dequantize(self, packed: torch.Tensor, divide_by: float | None = None) -> None:
+        """Dequantizes ``packed`` into the tensors; with ``divide_by`` they end up with the
+        bytes of dequantizing and then dividing each of them by that Python number."""
+        plan = self.plan
+        _check_packed(packed, plan, self.device)
+        raw = _stream_of(self.device)
+        tensors, table, pointers = self._ptrs, None, None
+        if self._table is not None:
+            tensors = None
+            table, pointers = self._long_list_args(raw, True)
+        if divide_by is None:
+            _check(self._lib.tftq_dequantize(self._handle, tensors, table, pointers, packed.data_ptr(),
+                                             plan.output_size, self._dev_index, raw), "tftq_dequantize")
+        else:
+            # torch divides a GPU tensor by a host scalar as a multiplication by the
+            # reciprocal, computed in double and rounded to fp32
+            divisor = float(divide_by)
+            factor = 1.0 / divisor if divisor != 0.0 else math.copysign(math.inf, divisor)
+            _check(self._lib.tftq_dequantize_scaled(self._handle, tensors, table, pointers, packed.data_ptr(),
+                                                    plan.output_size, factor, self._dev_index, raw),
+                   "tftq_dequantize_scaled")
 
 
 def _check_packed(output: torch.Tensor, plan: _Plan, device: torch.device) -> None:
@@ -212,49 +336,33 @@ def _check_packed(output: torch.Tensor, plan: _Plan, device: torch.device) -> No
         raise RuntimeError(f"the packed buffer is on {output.device}, the tensors are on {device}")
 
 
-# The three stages on a prepared plan.  The public functions below prepare and
-# call these; torchft_amd.collectives prepares once per collective and calls
-# all three, which saves two walks over the tensor list.
-def _quantize(plan: _Plan, device: torch.device) -> torch.Tensor:
-    with _on_device(device):
-        # float32 storage like the reference (:567-571) so that scales are aligned
-        output = torch.empty(plan.output_size // SCALE_DTYPE_BYTES, device=device,
-                             dtype=SCALE_DTYPE).view(torch.uint8)
-        _check(plan._lib.tftq_quantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                       plan.output_size, _stream_ptr(device)), "tftq_quantize")
-        _keep_table(plan, device)
-    return output
-
-
-def _reduce(plan: _Plan, device: torch.device, output: torch.Tensor, rank: int,
-            reduce_op: ReduceOp) -> None:
-    _check_packed(output, plan, device)
-    is_avg = 0 if reduce_op == ReduceOp.SUM else 1  # anything but SUM averages (:682)
-    with _on_device(device):
-        _check(plan._lib.tftq_reduce(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                     plan.output_size, int(rank), is_avg,
-                                     _stream_ptr(device)), "tftq_reduce")
-        _keep_table(plan, device)
-
-
-def _dequantize(plan: _Plan, device: torch.device, output: torch.Tensor,
-                divide_by: float | None = None) -> None:
-    _check_packed(output, plan, device)
-    with _on_device(device):
-        if divide_by is None:
-            _check(plan._lib.tftq_dequantize(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                             plan.output_size, _stream_ptr(device)),
-                   "tftq_dequantize")
-        else:
-            # torch divides a GPU tensor by a host scalar as a multiplication by the
-            # reciprocal, computed in double and rounded to fp32
-            divisor = float(divide_by)
-            factor = 1.0 / divisor if divisor != 0.0 else math.copysign(math.inf, divisor)
-            _check(plan._lib.tftq_dequantize_scaled(plan.handle, ctypes.c_void_p(output.data_ptr()),
-                                                    plan.output_size, factor,
-                                                    _stream_ptr(device)),
-                   "tftq_dequantize_scaled")
-        _keep_table(plan, device)
+def prepare(inputs: list[torch.Tensor], all_reduce_group_size: int) -> PreparedBucket:
+    """Counterpart of ``_prepare_quantize_fp8`` (quantization.py:431-528): validates the
+    list, turns 1-D tensors into ``[k, 1]`` in the caller's list (:487-488), finds or
+    builds the plan for these shapes and binds the tensors' addresses to it.  This is the
+    only walk over the list; the returned bucket can be used any number of times."""
+    device, dtype = _validate(inputs)
+    if device.type != "cuda":
+        raise RuntimeError(
+            "torchft_amd.quantization needs tensors on a gfx950 GPU; there is no CPU path")
+    _lib.check_device(device.index)
+    ws = int(all_reduce_group_size)
+    T = len(inputs)
+    # The key holds tens of thousands of small tuples for long lists; keep the cyclic
+    # garbage collector from walking them while they are being built.
+    pause_gc = T > 256 and gc.isenabled()
+    if pause_gc:
+        gc.disable()
+    try:
+        sizes_key = tuple(map(_TENSOR.size, inputs))
+        strides_key = tuple(map(_TENSOR.stride, inputs))
+        plan = _plan_for(dtype, ws, sizes_key, strides_key)
+        ptrs = (ctypes.c_void_p * T)()
+        ptrs[:] = list(map(_TENSOR.data_ptr, inputs))
+    finally:
+        if pause_gc:
+            gc.enable()
+    return PreparedBucket(plan, device, list(inputs), ws, ptrs)
 
 
 def fused_quantize_into_fp8(
@@ -272,8 +380,7 @@ def fused_quantize_into_fp8(
     Returns:
         the packed uint8 tensor (``numel() % all_reduce_group_size == 0``)
     """
-    plan, device = _prepare(inputs, all_reduce_group_size)
-    return _quantize(plan, device)
+    return prepare(inputs, all_reduce_group_size).quantize()
 
 
 def fused_dequantize_from_fp8(
@@ -290,8 +397,7 @@ def fused_dequantize_from_fp8(
     up with the bytes that dequantizing and then dividing each of them by that
     Python number on the GPU gives.
     """
-    plan, device = _prepare(inputs, all_reduce_group_size)
-    _dequantize(plan, device, output, divide_by)
+    prepare(inputs, all_reduce_group_size).dequantize(output, divide_by)
 
 
 def fused_reduce_fp8(
@@ -307,5 +413,4 @@ def fused_reduce_fp8(
     Any ``reduce_op`` other than SUM averages (quantization.py:682).
     ``inputs`` only supplies the shapes.
     """
-    plan, device = _prepare(inputs, all_reduce_group_size)
-    _reduce(plan, device, output, all_reduce_rank, reduce_op)
+    prepare(inputs, all_reduce_group_size).reduce(output, all_reduce_rank, reduce_op)
