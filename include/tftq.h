@@ -65,6 +65,7 @@ extern "C" {
 #define TFTQ_E_NOMEM (-5)    /* host allocation failed */
 #define TFTQ_E_NOTABLE (-6)  /* a list longer than TFTQ_N_INLINE needs `table` (and `pointers`) */
 #define TFTQ_E_ARCH (-7)     /* the device is not gfx950 */
+#define TFTQ_E_TOOBIG (-8)   /* tftq_reduce_static: the list's table exceeds TFTQ_STATIC_TABLE_BYTES */
 
 typedef struct tftq_plan tftq_plan;
 
@@ -176,6 +177,26 @@ int tftq_dequantize(const tftq_plan *plan, void *const *tensors, const void *tab
 int tftq_dequantize_scaled(const tftq_plan *plan, void *const *tensors, const void *table,
                            void *pointers, const void *packed, int64_t packed_bytes,
                            float post_scale, int device, void *stream);
+
+/*
+ * tftq_reduce for callers that cannot hand over device memory for `table` and may not
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  For a long list the table image
+ * is written, with small kernels on `stream`, into a fixed array of
+ * TFTQ_STATIC_TABLE_BYTES bytes that the library's code object holds on every device
+ * it runs on, and the reduce kernel reads it from there; lists whose table is larger
+ * are refused with TFTQ_E_TOOBIG (90 to 190 bytes per tensor: lists of 2800 tensors always fit).
+ * Short lists use no scratch memory at all.  The call allocates and frees nothing; it
+ * costs one small kernel per 3584 bytes of table in front of the reduce kernel.  The
+ * array's address on a device is looked up once, by tftq_check_device() for that device
+ * or else by the first call there (which should then not run under stream capture).
+ * All calls on one device share that array: calls that overlap in time on one device
+ * (different streams or threads) race on it and must be serialised by the caller.
+ * Results are those of tftq_reduce.
+ */
+#define TFTQ_STATIC_TABLE_BYTES (512 * 1024)
+int tftq_reduce_static(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank,
+                       int is_avg, int device, void *stream);
 
 #ifdef __cplusplus
 }

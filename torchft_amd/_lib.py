@@ -13,7 +13,7 @@ _lib: ctypes.CDLL | None = None
 
 ERR_NAMES = {
     -1: "TFTQ_E_ARG", -2: "TFTQ_E_DTYPE", -3: "TFTQ_E_SHAPE", -4: "TFTQ_E_SIZE",
-    -5: "TFTQ_E_NOMEM", -6: "TFTQ_E_NOTABLE", -7: "TFTQ_E_ARCH",
+    -5: "TFTQ_E_NOMEM", -6: "TFTQ_E_NOTABLE", -7: "TFTQ_E_ARCH", -8: "TFTQ_E_TOOBIG",
 }
 
 # every symbol that include/tftq.h declares: (name, restype, argtypes)
@@ -43,6 +43,8 @@ SYMBOLS = [
     ("tftq_reduce", _c.c_int, [_P, _P, _P, _c.c_int64, _c.c_int, _c.c_int, _c.c_int, _P]),
     ("tftq_dequantize", _c.c_int, [_P, _P, _P, _P, _P, _c.c_int64, _c.c_int, _P]),
     ("tftq_dequantize_scaled", _c.c_int, [_P, _P, _P, _P, _P, _c.c_int64, _c.c_float, _c.c_int, _P]),
+    # plan, packed, packed_bytes, rank, is_avg, device, stream
+    ("tftq_reduce_static", _c.c_int, [_P, _P, _c.c_int64, _c.c_int, _c.c_int, _c.c_int, _P]),
 ]
 ABI_VERSION = 2
 

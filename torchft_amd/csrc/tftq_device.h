@@ -498,6 +498,10 @@ struct DeviceScope {
 __attribute__((visibility("hidden"))) int tftq_put_bytes(void *dst_device, const void *src_host, size_t bytes,
                                                          hipStream_t st);
 
+// Looks up, for the current device, the address of the fixed array that tftq_reduce_static
+// keeps its table in.  Defined in tftq_reduce.hip.
+__attribute__((visibility("hidden"))) int tftq_static_table_setup(void);
+
 // One kernel launch with the launch's own error (not whatever an earlier call left behind).
 template <typename K>
 static inline int launch_kernel(K kernel, unsigned grid, unsigned lds_bytes, hipStream_t st, const KParams &kp,

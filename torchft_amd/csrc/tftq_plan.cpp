@@ -36,6 +36,7 @@ extern "C" const char *tftq_strerror(int code)
     case TFTQ_E_NOMEM: return "out of host memory";
     case TFTQ_E_NOTABLE: return "a list of more than 16 tensors needs the device table and the pointer buffer";
     case TFTQ_E_ARCH: return "device is not gfx950";
+    case TFTQ_E_TOOBIG: return "the list's descriptor table does not fit the library's fixed array";
     default: return code > 0 ? "HIP error" : "unknown error";
     }
 }

@@ -2,6 +2,8 @@
 //
 // Follows torchft/quantization.py:261-428 (kernels) and :638-686 (launcher); design notes in tftq_device.h.
 
+#include <mutex>
+
 #include "tftq_device.h"
 
 // ---------------------------------------------------------------------------
@@ -922,4 +924,64 @@ extern "C" int tftq_reduce(const tftq_plan *plan, const void *table, void *packe
     DeviceScope scope(device);
     if (scope.err != hipSuccess) return (int)scope.err;
     return reduce_launch(plan, table, packed, packed_bytes, rank, is_avg, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------
+// tftq_reduce_static: the descriptor table in a fixed array of the code object
+// ---------------------------------------------------------------------------
+// Every device the library runs on holds its own copy of this array at its own address.
+// Host code never uses the array's name as an address: it asks the runtime for the address
+// on the current device once (static_table_address) and uses that pointer from then on.
+static __device__ __align__(256) uint8_t static_table[TFTQ_STATIC_TABLE_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static void *static_table_ptr[MAX_DEVICES];  // per device ordinal; 0 = not looked up yet
+static std::mutex static_table_mutex;
+
+// Address of static_table on the device that is current on the calling thread.
+static int static_table_address(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return TFTQ_E_ARG;
+    std::lock_guard<std::mutex> guard(static_table_mutex);
+    if (!static_table_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_table));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return TFTQ_E_ARG;
+        static_table_ptr[dev] = p;
+    }
+    *out = static_table_ptr[dev];
+    return 0;
+}
+
+// Set-up for the current device (called by tftq_check_device).
+int tftq_static_table_setup(void)
+{
+    void *p = nullptr;
+    return static_table_address(&p);
+}
+
+extern "C" int tftq_reduce_static(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank, int is_avg,
+                                  int device, void *stream)
+{
+    if (!plan) return TFTQ_E_ARG;
+    DeviceScope scope(device);
+    if (scope.err != hipSuccess) return (int)scope.err;
+    hipStream_t st = (hipStream_t)stream;
+    if (plan->nseg <= TFTQ_N_INLINE || plan->nwg[ST_R] == 0)  // descriptors in the kernel arguments: no scratch
+        return reduce_launch(plan, nullptr, packed, packed_bytes, rank, is_avg, st);
+    if (plan->blob.size() > (size_t)TFTQ_STATIC_TABLE_BYTES) return TFTQ_E_TOOBIG;
+    if (packed_bytes != plan->output_size) return TFTQ_E_SIZE;  // before anything is queued
+    if (rank < 0 || rank >= plan->ws || (!packed && plan->output_size != 0) || ((uintptr_t)packed & 3) != 0)
+        return TFTQ_E_ARG;
+    void *table = nullptr;
+    int rc = static_table_address(&table);
+    if (rc) return rc;
+    // the whole image every time: the array keeps whatever the last call, of any plan, left there
+    rc = tftq_put_bytes(table, plan->blob.data(), plan->blob.size(), st);
+    if (rc) return rc;
+    return reduce_launch(plan, table, packed, packed_bytes, rank, is_avg, st);
 }

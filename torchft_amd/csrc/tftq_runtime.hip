@@ -53,7 +53,8 @@ extern "C" int tftq_check_device(int device)
     e = hipGetDeviceProperties(&prop, dev);
     if (e != hipSuccess) return (int)e;
     const char *a = prop.gcnArchName;
-    return (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')
-               ? 0
-               : TFTQ_E_ARCH;
+    if (!(a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')) return TFTQ_E_ARCH;
+    DeviceScope scope(dev);
+    if (scope.err != hipSuccess) return (int)scope.err;
+    return tftq_static_table_setup();
 }
