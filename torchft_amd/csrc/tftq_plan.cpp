@@ -131,11 +131,12 @@ static void work_order(const tftq_plan *p, int st, std::vector<int32_t> &ord)
 // natural order (4096 bf16 columns 122.0 -> 117.9 us, 14336: 122.4 -> 115.7, 256: 148.0 ->
 // 140.4, 4096 fp32: 101.4 -> 96.3) when the tensor rows are whole 64-byte blocks, and 5 %
 // slower when they are not (1000 columns: neighbouring rows then share blocks across XCDs);
-// quantize gains 2.5 % for fp32 tensors and loses up to 2 % for 16-bit ones; reduce does not care
-// and keeps the eighths, which its heaviest-first order is built on.
+// quantize, which writes its packed rows as whole lines from LDS, gains 2 % (benchmark
+// configuration 3: 114.0 -> 111.6 us); reduce does not care and keeps the eighths, which
+// its heaviest-first order is built on.
 static bool natural_order(const tftq_plan *p, int st)
 {
-    if (st == ST_R || (st == ST_Q && p->esz != 4)) return false;
+    if (st == ST_R) return false;
     double whole = 0.0, all = 0.0;
     for (int i = 0; i < p->nseg; i++) {
         const Seg &s = p->segs[(size_t)i];

@@ -20,18 +20,57 @@ DEV float vec_absmax(const u32x4 v)
     return a;
 }
 
+// the 4 (fp32) or 8 (16-bit) codes of one input vector: one or two dwords
 template <typename T>
-DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
+DEV u32x2 vec_codes(const u32x4 v, float s)
 {
     float f[Elem<T>::EPV];
     Elem<T>::unpack(v, f);
+    u32x2 o = {0u, 0u};
+    o.x = pack_fp8x4(f[0] * s, f[1] * s, f[2] * s, f[3] * s);
+    if constexpr (Elem<T>::EPV == 8) o.y = pack_fp8x4(f[4] * s, f[5] * s, f[6] * s, f[7] * s);
+    return o;
+}
+
+template <typename T>
+DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
+{
+    const u32x2 o = vec_codes<T>(v, s);
     if constexpr (Elem<T>::EPV == 4) {
-        payload[idx] = pack_fp8x4(f[0] * s, f[1] * s, f[2] * s, f[3] * s);
+        payload[idx] = o.x;
     } else {
-        u32x2 o;
-        o.x = pack_fp8x4(f[0] * s, f[1] * s, f[2] * s, f[3] * s);
-        o.y = pack_fp8x4(f[4] * s, f[5] * s, f[6] * s, f[7] * s);
         *(GLOBAL u32x2_a4 *)(payload + 2 * idx) = o;  // plain store: rows start 4 bytes off a line, L2 merges
+    }
+}
+
+// Staging of a workgroup's packed rows in LDS.  The rows that one workgroup quantizes are
+// neighbours in the packed buffer, so together they are one span of bytes; packed rows
+// start anywhere (4 + n bytes each), which makes direct stores cover parts of 128-byte
+// lines with every instruction.  The workgroup instead assembles the span in LDS, at the
+// offset that the span has inside its first 128-byte line, and then copies it out with
+// streaming 16-byte stores whose wavefronts each cover eight whole lines; only the first
+// and the last 16 bytes of the span can be partial and go out as dwords.
+constexpr int Q_STAGE_BYTES = 16640;  // 8 rows of 2052 bytes (2048 16-bit columns) + 127 bytes of offset, rounded up
+#define LDS_AS __attribute__((address_space(3)))
+
+DEV void copy_out_span(const uint8_t *stage, uint8_t *g0, int len, int tid)
+{
+    const int mis = (int)((uintptr_t)g0 & 127u);
+    GLOBAL uint8_t *line0 = as_global<uint8_t>(g0 - mis);  // stage[x] belongs at line0[x]
+    const int end = mis + len;
+    const int nchunks = (end + 15) >> 4;
+#pragma nounroll
+    for (int c = tid; c < nchunks; c += TFTQ_WG) {
+        const int lo = 16 * c;
+        const u32x4 v = *(const LDS_AS u32x4 *)(const LDS_AS uint8_t *)(stage + lo);
+        if (lo >= mis && lo + 16 <= end) {
+            STORE_STREAM(v, (GLOBAL u32x4 *)(line0 + lo));
+        } else {  // the span's first or last 16 bytes
+            const u32 w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                if (lo + 4 * d >= mis && lo + 4 * d < end) *(GLOBAL u32 *)(line0 + lo + 4 * d) = w[d];
+        }
     }
 }
 
@@ -39,16 +78,20 @@ DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
 // loads of a lane are issued back to back without a branch in between: lanes
 // past the end of the row re-read its last vector (a duplicate cannot change
 // the maximum) and simply do not store.
-template <typename T, int TEAM, int KMAX>
-DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float *lds)
+// STAGED: the row is a real one and its packed image goes to LDS at srow (see copy_out_span).
+template <typename T, int TEAM, int KMAX, bool STAGED = false>
+DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float *lds, LDS_AS u32 *srow = nullptr)
 {
-    const bool active = row < s.slice_rows * p.ws;
-    GLOBAL u32 *out = as_global<u32>(p.packed + (active ? row_addr(s, p.slot_size, row) : 0));
-    if (active && row >= s.m) {
-        // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
-        for (int d = lane; d < (s.row_bytes >> 2); d += TEAM) out[d] = 0;
+    GLOBAL u32 *out = nullptr;
+    if (!STAGED) {
+        const bool active = row < s.slice_rows * p.ws;
+        out = as_global<u32>(p.packed + (active ? row_addr(s, p.slot_size, row) : 0));
+        if (active && row >= s.m) {
+            // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
+            for (int d = lane; d < (s.row_bytes >> 2); d += TEAM) out[d] = 0;
+        }
+        if (!active || row >= s.m) return;  // a team leaves whole: its lanes share the row
     }
-    if (!active || row >= s.m) return;  // a team leaves whole: its lanes share the row
 
     constexpr int EPV = Elem<T>::EPV;
     const int nvec = s.n / EPV;
@@ -72,7 +115,10 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     }
     amax = team_max<TEAM>(amax, lds);
     const float sc = calc_scale(amax);
-    if (lane == 0) out[0] = as_u(sc);
+    if (lane == 0) {
+        if (STAGED) srow[0] = as_u(sc);
+        else out[0] = as_u(sc);
+    }
     // The elements are unpacked again from the raw vectors: keeping the floats of the
     // maximum search alive until here would double the registers of 16-bit inputs.
 #pragma unroll
@@ -80,20 +126,34 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
 #pragma unroll
     for (int k = 0; k < KMAX; k++) {
         const int idx = k * TEAM + lane;
-        if (idx < nvec) vec_quant_store<T>(v[k], sc, out + 1, idx);
+        if (idx < nvec) {
+            if (STAGED) {
+                const u32x2 o = vec_codes<T>(v[k], sc);
+                if constexpr (EPV == 4) {
+                    srow[1 + idx] = o.x;
+                } else {
+                    srow[1 + 2 * idx] = o.x;
+                    srow[2 + 2 * idx] = o.y;
+                }
+            } else {
+                vec_quant_store<T>(v[k], sc, out + 1, idx);
+            }
+        }
     }
     if (tail && lane == 0) {
         float y[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) y[e] = (e < EPV - 1 && e < tail) ? t[e < EPV - 1 ? e : 0] * sc : 0.0f;
-        GLOBAL u32 *tw = out + 1 + nvec * (EPV / 4);
+        const int td = 1 + nvec * (EPV / 4);  // dword of the row that holds the first tail code
         u32 w0 = pack_fp8x4(y[0], y[1], y[2], y[3]);
         if (tail < 4) w0 &= (1u << (8 * tail)) - 1u;  // padding bytes are zero whatever 0 * sc gave
-        tw[0] = w0;
+        if (STAGED) srow[td] = w0;
+        else out[td] = w0;
         if (EPV == 8 && tail > 4) {
             u32 w1 = pack_fp8x4(y[4], y[5], y[6], y[7]);
             if (tail < 8) w1 &= (1u << (8 * (tail - 4))) - 1u;
-            tw[1] = w1;
+            if (STAGED) srow[td + 1] = w1;
+            else out[td + 1] = w1;
         }
     }
 }
@@ -212,6 +272,38 @@ DEV void quantize_vec(const Seg &s, const KParams &p, int row, int lane, float *
     else if (WIDE && nvec <= TFTQ_Q_VECS_WIDE) quantize_vec_k<T, TEAM, 2 * QV>(s, p, row, lane, lds);
     else if (WIDE) quantize_vec_lds<T>(s, p, row, lane, lds, park);
     // else: the planner launches the wide kernel, with its LDS, for plans that have such rows
+}
+
+// The TFTQ_WG / TEAM rows of workgroup blk.  When they are all real rows of one slot (all
+// but the workgroups at the end of a slot or of the tensor) and fit the staging buffer,
+// their packed rows are assembled in LDS and written as one span; otherwise row by row.
+template <typename T, int TEAM, bool WIDE>
+DEV void quantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, float *lds, u32x4 *park, uint8_t *stage)
+{
+    constexpr int R = TFTQ_WG / TEAM;
+    const int r0 = blk * R;
+    const int team = TEAM == 64 ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid / TEAM;
+    const int lane = tid & (TEAM - 1);
+    if constexpr (!WIDE) {
+        const int nvec = s.n / Elem<T>::EPV;
+        const int last = r0 + R - 1;
+        if (last < s.m && nvec <= QV * TEAM) {
+            const int slot = r0 / s.slice_rows;
+            const int j = r0 - slot * s.slice_rows;
+            uint8_t *g0 = p.packed + (int64_t)slot * p.slot_size + s.slot_off + (int64_t)j * s.row_bytes;
+            const int mis = (int)((uintptr_t)g0 & 127u);
+            const int len = R * s.row_bytes;
+            if (j + R <= s.slice_rows && mis + len <= Q_STAGE_BYTES) {  // same for the whole workgroup
+                LDS_AS u32 *srow = (LDS_AS u32 *)(LDS_AS uint8_t *)(stage + mis + team * s.row_bytes);
+                if (nvec <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2, true>(s, p, r0 + team, lane, lds, srow);
+                else quantize_vec_k<T, TEAM, QV, true>(s, p, r0 + team, lane, lds, srow);
+                __syncthreads();
+                copy_out_span(stage, g0, len, tid);
+                return;
+            }
+        }
+    }
+    quantize_vec<T, TEAM, WIDE && TEAM == 256>(s, p, r0 + team, lane, lds, park);
 }
 
 // Any strides, any alignment, any n: element loads, two passes over the row
@@ -392,6 +484,7 @@ template <typename T, bool INLINE, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
+    __shared__ __align__(16) uint8_t stage[WIDE ? 16 : Q_STAGE_BYTES];  // see copy_out_span
     // 60 KB of dynamic LDS, asked for at the launch only when the plan has rows that need it
     // (it limits a CU to two workgroups)
     extern __shared__ u32x4 park[];
@@ -401,13 +494,11 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
     const int blk = vb - s.wg_begin[ST_Q];
     const int tid = threadIdx.x;
     switch (s.kind[ST_Q]) {
-    case K_VEC256: quantize_vec<T, 256, WIDE>(s, p, blk, tid, lds, park); break;
-    case K_VEC64:
-        quantize_vec<T, 64, false>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63, lds, park);
-        break;
-    case K_VEC32: quantize_vec<T, 32, false>(s, p, blk * 8 + (tid >> 5), tid & 31, lds, park); break;
-    case K_VEC16: quantize_vec<T, 16, false>(s, p, blk * 16 + (tid >> 4), tid & 15, lds, park); break;
-    case K_VEC8: quantize_vec<T, 8, false>(s, p, blk * 32 + (tid >> 3), tid & 7, lds, park); break;
+    case K_VEC256: quantize_vec_rows<T, 256, WIDE>(s, p, blk, tid, lds, park, stage); break;
+    case K_VEC64: quantize_vec_rows<T, 64, WIDE>(s, p, blk, tid, lds, park, stage); break;
+    case K_VEC32: quantize_vec_rows<T, 32, WIDE>(s, p, blk, tid, lds, park, stage); break;
+    case K_VEC16: quantize_vec_rows<T, 16, WIDE>(s, p, blk, tid, lds, park, stage); break;
+    case K_VEC8: quantize_vec_rows<T, 8, WIDE>(s, p, blk, tid, lds, park, stage); break;
     case K_GEN64:
         quantize_gen<T, 64>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;
