@@ -43,36 +43,7 @@ DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
     }
 }
 
-// Staging of a workgroup's packed rows in LDS.  The rows that one workgroup quantizes are
-// neighbours in the packed buffer, so together they are one span of bytes; packed rows
-// start anywhere (4 + n bytes each), which makes direct stores cover parts of 128-byte
-// lines with every instruction.  The workgroup instead assembles the span in LDS, at the
-// offset that the span has inside its first 128-byte line, and then copies it out with
-// streaming 16-byte stores whose wavefronts each cover eight whole lines; only the first
-// and the last 16 bytes of the span can be partial and go out as dwords.
-constexpr int Q_STAGE_BYTES = 16640;  // 8 rows of 2052 bytes (2048 16-bit columns) + 127 bytes of offset, rounded up
-#define LDS_AS __attribute__((address_space(3)))
-
-DEV void copy_out_span(const uint8_t *stage, uint8_t *g0, int len, int tid)
-{
-    const int mis = (int)((uintptr_t)g0 & 127u);
-    GLOBAL uint8_t *line0 = as_global<uint8_t>(g0 - mis);  // stage[x] belongs at line0[x]
-    const int end = mis + len;
-    const int nchunks = (end + 15) >> 4;
-#pragma nounroll
-    for (int c = tid; c < nchunks; c += TFTQ_WG) {
-        const int lo = 16 * c;
-        const u32x4 v = *(const LDS_AS u32x4 *)(const LDS_AS uint8_t *)(stage + lo);
-        if (lo >= mis && lo + 16 <= end) {
-            STORE_STREAM(v, (GLOBAL u32x4 *)(line0 + lo));
-        } else {  // the span's first or last 16 bytes
-            const u32 w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-                if (lo + 4 * d >= mis && lo + 4 * d < end) *(GLOBAL u32 *)(line0 + lo + 4 * d) = w[d];
-        }
-    }
-}
+constexpr int Q_STAGE_BYTES = 16640;  // 8 rows of 2052 bytes (2048 16-bit columns) + 127 bytes of offset, rounded up (see copy_out_span)
 
 // Contiguous, 16-byte aligned rows of at most TEAM * KMAX vectors.  The KMAX
 // loads of a lane are issued back to back without a branch in between: lanes

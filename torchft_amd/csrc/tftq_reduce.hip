@@ -818,7 +818,8 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
             // (10240 columns: 3, 3, 2, 2 instead of 3 each: 55.0 -> 50.4 us on [20480, 10240]).
             // Every variant passes the team's barriers the same number of times.
             const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-            const int nu = min((ndw + 1023) >> 10, (ndw - 256 * wave + 1023) >> 10);
+            // (at least one: a wavefront past the end of a short row still takes part in the barriers)
+            const int nu = max(1, min((ndw + 1023) >> 10, (ndw - 256 * wave + 1023) >> 10));
             if (nu == 1) reduce_rows<256, 1, true, GDIV>(s, p, j, tid, lds);
             // rows of three or four vectors per lane run the rolling window in all their wavefronts
             // ([20480, 10240]: 53.5 -> 50.4 us against the pipeline in the upper two); rows of two
