@@ -553,6 +553,14 @@ def test_cfg3_full_size(q, oracle):
     q.fused_reduce_fp8(list(peers_gpu[0]), recv, ws, rank, ReduceOp.AVG)
     oracle.fused_reduce_fp8(list(peer0_cpu), recv_cpu, ws, rank, ReduceOp.AVG, nthreads=NT)
     same_bytes(recv, recv_cpu, "cfg3 reduce rank 5")
+    # dequantize of that whole buffer (one reduced slot, seven as received), every tensor by bytes
+    outs = [torch.empty_like(t) for t in peers_gpu[0]]
+    outs_cpu = [torch.empty_like(t) for t in peer0_cpu]
+    q.fused_dequantize_from_fp8(outs, recv, ws)
+    oracle.fused_dequantize_from_fp8(outs_cpu, recv_cpu, ws, nthreads=NT)
+    for i, (a, b) in enumerate(zip(outs, outs_cpu)):
+        same_bytes(a, b, f"cfg3 dequantize tensor {i}")
+    del outs_cpu, recv_cpu
     # round trip of peer 0 alone: quantize -> dequantize is within half an fp8 ULP per row
     outs = [torch.empty_like(t) for t in peers_gpu[0]]
     q.fused_dequantize_from_fp8(outs, qs[0], ws)
@@ -634,6 +642,40 @@ def test_cfg4_full_size(q, oracle):
         amax = x.abs().amax(dim=1, keepdim=True)
         tol = torch.maximum(x.abs() * 2 ** -4, amax * (2 ** -10 / 448.0)) * 1.001
         assert ((x - o).abs() <= tol).all()
+    del outs
+
+    # One rank's reduction of four different peers and the dequantization of the result, at
+    # full size on the GPU; the picked tensors byte for byte against the checker, which works
+    # on single-tensor buffers cut out of the full ones (a tensor's rows sit at the same
+    # offsets in every slot, so its ws row slices are a packed buffer of that tensor alone).
+    recv = torch.empty_like(packed)
+    recv[rank * slot:(rank + 1) * slot] = packed[rank * slot:(rank + 1) * slot]
+    del packed
+    for p in range(ws):
+        if p == rank:
+            continue
+        other = workloads.cfg4(p, device="cuda")
+        qp = q.fused_quantize_into_fp8(other, ws)
+        recv[p * slot:(p + 1) * slot] = qp[rank * slot:(rank + 1) * slot]
+        del other, qp
+    received = recv.clone()
+    q.fused_reduce_fp8(mine, recv, ws, rank, ReduceOp.AVG)
+    outs = [torch.empty_like(t) for t in mine]
+    q.fused_dequantize_from_fp8(outs, recv, ws)
+    for i in picks:
+        m, n = shapes[i]
+        sr, rb = -(-m // ws), (-(-n // 4) + 1) * 4
+
+        def cut(buf):
+            return torch.cat([buf[p * slot + offs[i]: p * slot + offs[i] + sr * rb] for p in range(ws)]).cpu()
+
+        like = torch.empty(m, n)
+        mini = cut(received)
+        oracle.fused_reduce_fp8([like], mini, ws, rank, ReduceOp.AVG, nthreads=NT)
+        same_bytes(cut(recv), mini, f"cfg4 reduce tensor {i}")
+        want = [torch.empty(m, n)]
+        oracle.fused_dequantize_from_fp8(want, mini, ws, nthreads=NT)
+        same_bytes(outs[i], want[0], f"cfg4 dequantize tensor {i}")
 
 
 def test_cfg5_full_size(q, oracle):
