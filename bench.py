@@ -36,7 +36,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch on benchmark configuration 3 as profiled (profiles/cfg3_bf16_ws8_hbm_traffic.md)
-PROFILED_TRAFFIC = {"quantize": 655142000, "reduce": 246760000, "dequantize": 661483000}
+PROFILED_TRAFFIC = {"quantize": 655467519, "reduce": 247352320, "dequantize": 660080640}
 
 
 def parse_args():
