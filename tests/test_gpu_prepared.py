@@ -201,3 +201,27 @@ def test_persistent_buckets_equal_per_call_buckets(q, row_width):
             for i in range(len(sizes)):
                 same_bytes(results["persistent"][step][r][i], results["per_call"][step][r][i],
                            f"step {step} rank {r} tensor {i}")
+
+
+@pytest.mark.parametrize("n_tensors", [3, 40])
+def test_documented_binding(q, n_tensors):
+    """The minimal ctypes binding shown to maintainers runs as printed and gives the bytes of
+    the shipped wrapper, for a short list and for one that needs the device table; a second
+    call on fresh tensors of the same shapes reuses its plan."""
+    import os
+    import re
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "INTEGRATION.md")).read()
+    blocks = [b for b in re.findall(r"```python\n(.*?)```", text, flags=re.S) if "class Plan" in b]
+    assert len(blocks) == 1
+    code = blocks[0].replace('"torchft_amd/libtftq.so"', repr(os.path.join(root, "torchft_amd", "libtftq.so")))
+    scope: dict = {}
+    exec(compile(code, "documented_binding", "exec"), scope)
+    for seed in (1, 2):
+        tensors = make_list(n_tensors, seed)
+        got = scope["fused_quantize_into_fp8"](tensors, 4)
+        want = q.fused_quantize_into_fp8(tensors, 4)
+        torch.cuda.synchronize()
+        assert got.dtype == torch.uint8 and torch.equal(got, want)
+    assert len(scope["_plans"]) == 1
