@@ -107,14 +107,16 @@ def test_plan_errors():
 
 
 def test_plan_rejects_grids_the_hardware_cannot_launch():
-    """A grid has fewer than 2^32 threads = 2^24 workgroups of 256.  Rows of 600 fp32
-    columns are quantized by 32 lanes each, eight to a workgroup."""
-    rc, h = _plan(0, [(8 * (2 ** 24 - 64), 600)], [(600, 1)], 1)
+    """A grid has fewer than 2^32 threads = 2^24 workgroups of 256.  Rows of 640 fp32
+    columns are quantized and dequantized by 32 lanes each, eight to a workgroup."""
+    rc, h = _plan(0, [(8 * (2 ** 24 - 64), 640)], [(640, 1)], 1)
     assert rc == 0
     _lib.load().tftq_plan_destroy(h)
-    assert _plan(0, [(8 * 2 ** 24 + 64, 600)], [(600, 1)], 1)[0] == -3
+    assert _plan(0, [(8 * 2 ** 24 + 64, 640)], [(640, 1)], 1)[0] == -3
     # the same rows spread over 20 tensors (device table): rejected as well
-    assert _plan(0, [((8 * 2 ** 24) // 20 + 64, 600)] * 20, [(600, 1)] * 20, 1)[0] == -3
+    assert _plan(0, [((8 * 2 ** 24) // 20 + 64, 640)] * 20, [(640, 1)] * 20, 1)[0] == -3
+    # rows of 600 columns do not end on 64-byte boundaries: dequantize takes four to a workgroup
+    assert _plan(0, [(4 * 2 ** 24 + 64, 600)], [(600, 1)], 1)[0] == -3
 
 
 def test_host_wrapper_validation_messages():

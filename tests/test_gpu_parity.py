@@ -258,6 +258,58 @@ def test_unaligned_rows_and_tails(q, oracle, dtype):
             same_bytes(x, y, f"unaligned dequantize case {i} ws={ws}")  # guard elements included
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_dequantize_rows_through_lds_spans(q, oracle, dtype):
+    """Contiguous rows that do not start and end on 64-byte boundaries are dequantized into
+    LDS and written as one span per workgroup: row lengths on both sides of every team limit
+    (512 B, 1, 2, 4, 8, 16 KB), row counts that leave the last workgroup partly filled,
+    destinations at every dword offset inside a 128-byte line (and at odd element offsets,
+    which take the direct path), guard elements around every destination, and scales outside
+    the range of the fast division in some rows."""
+    g = torch.Generator().manual_seed(23)
+    esz = 4 if dtype == torch.float32 else 2
+    cases = []  # (m, n, element offset of the destination)
+    for row_bytes in (68, 500, 516, 1000, 1028, 2000, 2052, 3000, 4092, 4100, 6000, 8188, 8196, 12000, 16380, 16388):
+        n = row_bytes // esz
+        for m, off in ((37, 0), (9, 2 * (4 // esz)), (70, 30 * (4 // esz) + 64), (3, 1)):
+            cases.append((m, n, off))
+    cpu_src = []
+    for m, n, _ in cases:
+        t = torch.randn(m, n, generator=g) * 0.3
+        t[m // 2] *= 1e-30  # a scale beyond the fast division: plain divide in that row
+        if dtype == torch.float16:
+            t[m // 2] = 0.0
+            t[m // 2, 0] = 6e-8
+        cpu_src.append(t.to(dtype))
+    for ws in (1, 4):
+        b = oracle.fused_quantize_into_fp8(list(cpu_src), ws)
+        a = q.fused_quantize_into_fp8([t.cuda() for t in cpu_src], ws)
+        same_bytes(a, b, f"quantize ws={ws}")
+        out_c = [torch.full((m * n + off + 40,), 5.0, dtype=dtype) for m, n, off in cases]
+        out_g = [t.cuda() for t in out_c]
+        dst_c = [t[off:off + m * n].view(m, n) for t, (m, n, off) in zip(out_c, cases)]
+        dst_g = [t[off:off + m * n].view(m, n) for t, (m, n, off) in zip(out_g, cases)]
+        oracle.fused_dequantize_from_fp8(list(dst_c), b, ws)
+        q.fused_dequantize_from_fp8(list(dst_g), a, ws)
+        for i, (x, y) in enumerate(zip(out_g, out_c)):
+            same_bytes(x, y, f"dequantize case {cases[i]} ws={ws}")
+        if dtype == torch.float16:  # torch's own division does not treat the sign of fp16 zeros uniformly
+            continue
+        # the same rows as a short list (descriptors in the kernel arguments), with the division folded in
+        pick = list(range(5, len(cases), 7))[:12]
+        b2 = oracle.fused_quantize_into_fp8([cpu_src[i] for i in pick], ws)
+        a2 = q.fused_quantize_into_fp8([cpu_src[i].cuda() for i in pick], ws)
+        same_bytes(a2, b2, f"quantize short list ws={ws}")
+        o1 = [torch.full_like(dst_g[i], 3.0) for i in pick]
+        o2 = [torch.full_like(dst_g[i], 3.0) for i in pick]
+        q.fused_dequantize_from_fp8(o1, a2, ws)
+        for t in o1:
+            t /= 3
+        q.fused_dequantize_from_fp8(o2, a2, ws, divide_by=3)
+        for i, (x, y) in zip(pick, zip(o2, o1)):
+            same_bytes(x, y, f"dequantize with division case {cases[i]} ws={ws}")
+
+
 @pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (3, ReduceOp.AVG), (5, ReduceOp.SUM),
                                    (6, ReduceOp.AVG), (70, ReduceOp.AVG), (64, ReduceOp.SUM)])
 def test_group_sizes(q, oracle, ws, op):

@@ -7,15 +7,27 @@
 // ---------------------------------------------------------------------------
 // dequantize
 // ---------------------------------------------------------------------------
-// Streaming (nontemporal) stores pay off only when the pieces a store instruction
-// writes are whole 64-byte blocks: partial blocks written that way are not
-// merged in L2 (2000-byte bf16 rows: 3.5 TB/s streaming, 4.2 TB/s plain; 8000-byte
-// rows: 5.4 against 5.0).  True when the rows of the tensor start and end on
-// 64-byte boundaries.
+// Every store of dequantized values is a streaming (nontemporal) store.  Plain stores leave
+// their lines dirty in the memory-side cache, and whatever kernel runs next pays for the
+// write-back (a reduce launch behind a 436 MB dequantize with plain stores: 54-58 us instead
+// of 45 us, also after 200 us of idling).  Streaming stores pay off only when the pieces a
+// store instruction writes are whole 64-byte blocks: partial blocks written that way are not
+// merged in L2 (2000-byte bf16 rows written straight from the registers: 3.5 TB/s).  Rows that
+// do not start and end on 64-byte boundaries therefore go through LDS where they can
+// (dequantize_vec_rows), so that the workgroup writes whole 128-byte lines.
+// True when the rows of the tensor start and end on 64-byte boundaries.
 template <typename T>
 DEV bool rows_fill_lines(const Seg &s)
 {
     return ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ) | (uint64_t)((int64_t)s.n * Elem<T>::ESZ)) & 63u) == 0;
+}
+
+// one element into the LDS image of a row
+template <typename T>
+DEV void stage_elem(LDS_AS uint8_t *srow, int col, float v)
+{
+    if constexpr (Elem<T>::ESZ == 4) *(LDS_AS u32 *)(srow + 4 * col) = as_u(v);
+    else *(LDS_AS uint16_t *)(srow + 2 * col) = (uint16_t)(Elem<T>::pack2(v, 0.0f) & 0xFFFFu);
 }
 
 // The value that is stored: the quotient, or in the scaled variant (POST) the
@@ -56,9 +68,10 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
 // Contiguous rows.  DV vectors per lane and step; their loads are issued together
 // without a branch (lanes past the end re-read the last vector and do not store),
 // and the first step's loads are on their way before the row's scale has arrived
-// and been turned into division coefficients.
-template <typename T, int TEAM, bool NT, int DV, bool POST>
-DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
+// and been turned into division coefficients.  STAGED: the row is written to its
+// place in LDS (srow) instead of global memory.
+template <typename T, int TEAM, bool STAGED, int DV, bool POST>
+DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS_AS uint8_t *srow)
 {
     if (row >= s.m) return;
     GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
@@ -81,14 +94,24 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
     load_step(0);
     const DivCoef c = make_div(sraw);
     if (!c.fast) {  // same for all lanes of the team
-        dequantize_gen<T, TEAM, POST>(s, p, row, lane);
+        if constexpr (STAGED) {
+#pragma nounroll
+            for (int col = lane; col < s.n; col += TEAM) {
+                const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
+                stage_elem<T>(srow, col, fin<T, POST>(f / c.s, p));
+            }
+        } else {
+            dequantize_gen<T, TEAM, POST>(s, p, row, lane);
+        }
         return;
     }
     GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
     // the few columns after the last whole vector, one element per lane
     for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
         const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
-        Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p));
+        const float v = fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p);
+        if constexpr (STAGED) stage_elem<T>(srow, col, v);
+        else Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, v);
     }
     for (int base = 0;;) {
 #pragma unroll
@@ -105,8 +128,8 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
                 for (int e = 0; e < 4; e++) o[4 + e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
             }
             if (idx < nvec) {
-                if (NT) STORE_STREAM(Elem<T>::pack(o), out + idx);
-                else out[idx] = Elem<T>::pack(o);
+                if constexpr (STAGED) *(LDS_AS u32x4_a4 *)(srow + 16 * idx) = Elem<T>::pack(o);
+                else STORE_STREAM(Elem<T>::pack(o), out + idx);
             }
         }
         base += DV * TEAM;
@@ -115,20 +138,39 @@ DEV void dequantize_vec_nt(const Seg &s, const KParams &p, int row, int lane)
     }
 }
 
+// The 256 / TEAM rows of a workgroup.  Rows that start and end on 64-byte boundaries are
+// written straight from the registers.  Other rows, when they are contiguous in memory
+// (row stride = row length) and dword-aligned, make one span of bytes per workgroup, which
+// is assembled in LDS and written as whole lines (copy_out_span); that needs the span to fit
+// the stage, which the planner sees to for rows of up to 16 KB (pick_d_kind in tftq_plan.cpp).
+// What is left (longer rows, where the partial lines are few, and strided or oddly aligned
+// rows) is written from the registers, partial blocks included.
 template <typename T, int TEAM, bool POST>
-DEV void dequantize_vec(const Seg &s, const KParams &p, int row, int lane)
+DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
-    // same branch for the whole workgroup
+    constexpr int R = TFTQ_WG / TEAM;
+    const int r0 = blk * R;
+    const int team = TEAM == 256 ? 0 : TEAM >= 64 ? __builtin_amdgcn_readfirstlane(tid / TEAM) : tid / TEAM;
+    const int lane = tid & (TEAM - 1);
     // DV = vectors a lane loads per step: 8 in flight where the row has them (4 is 1.3 % slower
     // on 4096-column bf16 rows), 4 for shorter rows, whose lanes would mostly load duplicates
     const bool few = s.n / Elem<T>::EPV <= 4 * TEAM;
-    if (rows_fill_lines<T>(s)) {
-        if (few) dequantize_vec_nt<T, TEAM, true, 4, POST>(s, p, row, lane);
-        else dequantize_vec_nt<T, TEAM, true, 8, POST>(s, p, row, lane);
-    } else {
-        if (few) dequantize_vec_nt<T, TEAM, false, 4, POST>(s, p, row, lane);
-        else dequantize_vec_nt<T, TEAM, false, 8, POST>(s, p, row, lane);
+    const int64_t rowb = (int64_t)s.n * Elem<T>::ESZ;
+    // same branches for the whole workgroup
+    if (!rows_fill_lines<T>(s) && s.row_stride == s.n && ((s.ptr | (uint64_t)rowb) & 3u) == 0 &&
+        R * rowb + 127 <= TFTQ_D_STAGE) {
+        uint8_t *g0 = (uint8_t *)s.ptr + (int64_t)r0 * rowb;
+        const int mis = (int)((uintptr_t)g0 & 127u);
+        const int len = min(R, s.m - r0) * (int)rowb;
+        LDS_AS uint8_t *srow = (LDS_AS uint8_t *)stage + mis + team * (int)rowb;
+        if (few) dequantize_vec_k<T, TEAM, true, 4, POST>(s, p, r0 + team, lane, srow);
+        else dequantize_vec_k<T, TEAM, true, 8, POST>(s, p, r0 + team, lane, srow);
+        __syncthreads();
+        copy_out_span(stage, g0, len, tid);
+        return;
     }
+    if (few) dequantize_vec_k<T, TEAM, false, 4, POST>(s, p, r0 + team, lane, nullptr);
+    else dequantize_vec_k<T, TEAM, false, 8, POST>(s, p, r0 + team, lane, nullptr);
 }
 
 // Rows of one column: one plain divide per row.  Any element stride: four rows
@@ -282,19 +324,19 @@ DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid)
 template <typename T, bool INLINE, bool POST>
 __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const InlineTable inl)
 {
+    __shared__ __align__(16) uint8_t stage[TFTQ_D_STAGE];  // see copy_out_span
     Seg s;
     int vb;
     if (!locate<INLINE, ST_D>(p, inl, s, vb)) return;
     const int blk = vb - s.wg_begin[ST_D];
     const int tid = threadIdx.x;
     switch (s.kind[ST_D]) {
-    case K_VEC256: dequantize_vec<T, 256, POST>(s, p, blk, tid); break;
-    case K_VEC64:
-        dequantize_vec<T, 64, POST>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
-        break;
-    case K_VEC32: dequantize_vec<T, 32, POST>(s, p, blk * 8 + (tid >> 5), tid & 31); break;
-    case K_VEC16: dequantize_vec<T, 16, POST>(s, p, blk * 16 + (tid >> 4), tid & 15); break;
-    case K_VEC8: dequantize_vec<T, 8, POST>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
+    case K_VEC256: dequantize_vec_rows<T, 256, POST>(s, p, blk, tid, stage); break;
+    case K_VEC128: dequantize_vec_rows<T, 128, POST>(s, p, blk, tid, stage); break;
+    case K_VEC64: dequantize_vec_rows<T, 64, POST>(s, p, blk, tid, stage); break;
+    case K_VEC32: dequantize_vec_rows<T, 32, POST>(s, p, blk, tid, stage); break;
+    case K_VEC16: dequantize_vec_rows<T, 16, POST>(s, p, blk, tid, stage); break;
+    case K_VEC8: dequantize_vec_rows<T, 8, POST>(s, p, blk, tid, stage); break;
     case K_GEN64:
         dequantize_gen<T, 64, POST>(s, p, blk * 4 + __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
         break;

@@ -23,6 +23,7 @@ enum : uint8_t {
     K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
     K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
     K_VEC64 = 2,   // one wavefront per row, 4 rows per workgroup
+    K_VEC128 = 14, // two wavefronts per row, 2 rows per workgroup (dequantize only)
     K_VEC256 = 3,  // one workgroup per row (also loops over rows too long for registers)
     K_GEN1 = 4,    // one lane per row, 256 rows per workgroup
     K_GEN8 = 5,    // 8 lanes per row
@@ -47,6 +48,7 @@ TFTQ_HD static inline int tftq_team_of(uint8_t kind)
     case K_GEN16: case K_VEC16: return 16;
     case K_GEN32: case K_VEC32: return 32;
     case K_VEC64: case K_GEN64: return 64;
+    case K_VEC128: return 128;
     case K_VEC256: case K_GEN256: return 256;
     case K_GEN1: return 1;
     default: return 256;
@@ -116,6 +118,10 @@ constexpr int TFTQ_Q_VECS = 8 * TFTQ_WG, TFTQ_Q_VECS_WIDE = 16 * TFTQ_WG;
 constexpr int TFTQ_Q_PARKED = 15;  // more vectors per lane that the wide quantize kernel parks in LDS (60 KB)
 constexpr int TFTQ_Q_VECS_LDS = TFTQ_Q_VECS_WIDE + TFTQ_Q_PARKED * TFTQ_WG;
 constexpr int TFTQ_R_DWORDS = 4096, TFTQ_R_DWORDS_WIDE = 8192;
+// Dequantize assembles rows that do not fill their 64-byte blocks in LDS, one span of bytes
+// per workgroup, at the offset the span has in its first 128-byte line: 16 KB + 127 bytes,
+// rounded up, which leaves a CU all its workgroups.
+constexpr int TFTQ_D_STAGE = 16640;
 
 // One tensor of the list.  64 bytes.
 struct Seg {

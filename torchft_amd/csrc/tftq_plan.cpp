@@ -86,6 +86,24 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     return K_GEN64;
 }
 
+// Dequantize writes rows that do not start and end on 64-byte boundaries through LDS, one
+// span of 256 / team rows per workgroup (dequantize_vec_rows); the team is then the largest
+// whose rows fit the stage together.  Rows of more than 16 KB have few partial lines
+// and keep the team of pick_io_kind, as do rows that fill their lines.
+static uint8_t pick_d_kind(const Seg &s, int esz)
+{
+    const uint8_t k = pick_io_kind(s, esz);
+    const int64_t rowb = (int64_t)s.n * esz;
+    if (k != K_VEC8 && k != K_VEC16 && k != K_VEC32 && k != K_VEC64 && k != K_VEC256) return k;
+    if (s.row_stride != s.n || (rowb & 3) != 0 || (rowb & 63) == 0 || rowb > 16384) return k;
+    if (rowb <= 512) return K_VEC8;
+    if (rowb <= 1024) return K_VEC16;
+    if (rowb <= 2048) return K_VEC32;
+    if (rowb <= 4096) return K_VEC64;
+    if (rowb <= 8192) return K_VEC128;
+    return K_VEC256;
+}
+
 static uint8_t pick_reduce_kind(const Seg &s)
 {
     // one or two 16-byte vectors of codes per lane and peer, four for the longest rows
@@ -295,7 +313,8 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes,
         const int64_t m_pad = (int64_t)s.slice_rows * ws;
         if (m_pad > p->max_rows) p->max_rows = m_pad;
 
-        s.kind[ST_Q] = s.kind[ST_D] = pick_io_kind(s, p->esz);
+        s.kind[ST_Q] = pick_io_kind(s, p->esz);
+        s.kind[ST_D] = pick_d_kind(s, p->esz);
         s.kind[ST_R] = pick_reduce_kind(s);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
@@ -319,6 +338,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes,
         if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS_WIDE && s.m > 0) p->parked = true;
         if (s.kind[ST_R] == K_GEN256 && ndw > TFTQ_R_DWORDS && s.m > 0 && ws <= 64)
             p->wide[ST_R] = true;
+
     }
     try {
         if (p->nseg <= TFTQ_N_INLINE) deal_to_xcds(p, wgs);
