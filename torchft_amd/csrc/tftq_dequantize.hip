@@ -238,43 +238,26 @@ DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 
 // K_VECS in dequantize: same shape as quantize_small, 8 vectors of codes and their
 // rows' scales in flight per lane.
-template <typename T, int C, bool NT, bool POST>
-DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
+// Rows RBEG * teams .. REND * teams - 1 of the workgroup's rows.  STAGED: they are
+// neighbours in memory (row stride = row length) and go through the LDS stage as one span.
+template <typename T, int C, bool STAGED, bool POST, int RBEG, int REND>
+DEV void dequantize_small_rows(const Seg &s, const KParams &p, const SmallShape &h, const u32x2 (&w)[8 / C][C],
+                               const float (&sc)[8 / C], bool fast, int row0, uint8_t *stage, int tid)
 {
     constexpr int EPV = Elem<T>::EPV;
-    constexpr int ROWS = 8 / C;
     const int nvec = s.n / EPV;
-    const int row0 = blk * (h.teams * ROWS);
-    const float inv = 1.0f / (float)s.slice_rows;
-
-    u32x2 w[ROWS][C];
-    float sc[ROWS];
-    int row[ROWS];
+    const int rowb = nvec * 16;
+    const int last = min(row0 + h.teams * (8 / C), s.m) - 1;
+    const int first = row0 + RBEG * h.teams;
+    if (first > last) return;  // same for the whole workgroup
+    uint8_t *gp = (uint8_t *)s.ptr + (int64_t)first * rowb;  // used when STAGED
+    const int mis = (int)((uintptr_t)gp & 127u);
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        row[r] = row0 + r * h.teams + h.t;
-        GLOBAL const u32 *in =
-            as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, min(row[r], s.m - 1), inv));
-        sc[r] = as_f(in[0]);
-#pragma unroll
-        for (int k = 0; k < C; k++) {
-            const int idx = min(k * h.team + h.l, nvec - 1);
-            if constexpr (EPV == 4) {
-                w[r][k].x = LOAD_STREAM(in + 1 + idx);
-                w[r][k].y = 0;
-            } else {
-                w[r][k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
-            }
-        }
-    }
-    bool all_fast = true;
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) all_fast = all_fast && scale_is_fast(sc[r]);
-    const bool fast = __builtin_amdgcn_ballot_w64(!all_fast) == 0;  // one code path per wavefront
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
+    for (int r = RBEG; r < REND; r++) {
+        const int row = row0 + r * h.teams + h.t;
         const DivCoef c = make_div(sc[r]);
-        GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)min(row[r], s.m - 1) * s.row_stride * Elem<T>::ESZ);
+        GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)min(row, s.m - 1) * s.row_stride * Elem<T>::ESZ);
+        LDS_AS uint8_t *srow = (LDS_AS uint8_t *)stage + mis + ((r - RBEG) * h.teams + h.t) * rowb;
 #pragma unroll
         for (int k = 0; k < C; k++) {
             float f[4], g[4], o[EPV];
@@ -296,28 +279,70 @@ DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, co
                 }
             }
             const int vec = k * h.team + h.l;
-            if (row[r] < s.m && vec < nvec) {
-                if (NT) STORE_STREAM(Elem<T>::pack(o), out + vec);
-                else out[vec] = Elem<T>::pack(o);
+            if (row < s.m && vec < nvec) {
+                if constexpr (STAGED) *(LDS_AS u32x4_a4 *)(srow + 16 * vec) = Elem<T>::pack(o);
+                else STORE_STREAM(Elem<T>::pack(o), out + vec);
             }
         }
     }
+    if constexpr (STAGED) {
+        __syncthreads();
+        copy_out_span(stage, gp, (min(last, row0 + REND * h.teams - 1) - first + 1) * rowb, tid);
+    }
+}
+
+template <typename T, int C, bool STAGED, bool POST>
+DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int ROWS = 8 / C;  // 8, 4 or 2
+    const int nvec = s.n / EPV;
+    const int row0 = blk * (h.teams * ROWS);
+    const float inv = 1.0f / (float)s.slice_rows;
+
+    u32x2 w[ROWS][C];
+    float sc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const int row = row0 + r * h.teams + h.t;
+        GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, min(row, s.m - 1), inv));
+        sc[r] = as_f(in[0]);
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            const int idx = min(k * h.team + h.l, nvec - 1);
+            if constexpr (EPV == 4) {
+                w[r][k].x = LOAD_STREAM(in + 1 + idx);
+                w[r][k].y = 0;
+            } else {
+                w[r][k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
+            }
+        }
+    }
+    bool all_fast = true;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) all_fast = all_fast && scale_is_fast(sc[r]);
+    const bool fast = __builtin_amdgcn_ballot_w64(!all_fast) == 0;  // one code path per wavefront
+    // a workgroup writes up to 32 KB: two halves through the stage
+    dequantize_small_rows<T, C, STAGED, POST, 0, ROWS / 2>(s, p, h, w, sc, fast, row0, stage, tid);
+    if constexpr (STAGED) __syncthreads();  // the first half has been copied out of the stage
+    dequantize_small_rows<T, C, STAGED, POST, ROWS / 2, ROWS>(s, p, h, w, sc, fast, row0, stage, tid);
 }
 
 template <typename T, bool POST>
-DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid)
+DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
     const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
-    if (rows_fill_lines<T>(s)) {
-        if (h.c == 1) dequantize_small_c<T, 1, true, POST>(s, p, blk, tid, h);
-        else if (h.c == 2) dequantize_small_c<T, 2, true, POST>(s, p, blk, tid, h);
-        else if (h.c == 3) dequantize_small_c<T, 3, true, POST>(s, p, blk, tid, h);
-        else dequantize_small_c<T, 4, true, POST>(s, p, blk, tid, h);
+    // same branch for the whole workgroup
+    if (!rows_fill_lines<T>(s) && s.row_stride == s.n && (s.ptr & 3u) == 0) {
+        if (h.c == 1) dequantize_small_c<T, 1, true, POST>(s, p, blk, tid, h, stage);
+        else if (h.c == 2) dequantize_small_c<T, 2, true, POST>(s, p, blk, tid, h, stage);
+        else if (h.c == 3) dequantize_small_c<T, 3, true, POST>(s, p, blk, tid, h, stage);
+        else dequantize_small_c<T, 4, true, POST>(s, p, blk, tid, h, stage);
     } else {
-        if (h.c == 1) dequantize_small_c<T, 1, false, POST>(s, p, blk, tid, h);
-        else if (h.c == 2) dequantize_small_c<T, 2, false, POST>(s, p, blk, tid, h);
-        else if (h.c == 3) dequantize_small_c<T, 3, false, POST>(s, p, blk, tid, h);
-        else dequantize_small_c<T, 4, false, POST>(s, p, blk, tid, h);
+        if (h.c == 1) dequantize_small_c<T, 1, false, POST>(s, p, blk, tid, h, stage);
+        else if (h.c == 2) dequantize_small_c<T, 2, false, POST>(s, p, blk, tid, h, stage);
+        else if (h.c == 3) dequantize_small_c<T, 3, false, POST>(s, p, blk, tid, h, stage);
+        else dequantize_small_c<T, 4, false, POST>(s, p, blk, tid, h, stage);
     }
 }
 
@@ -345,7 +370,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_dequantize(const KParams p, const I
     case K_COL1:
         if (s.m > 0) dequantize_col1<T, POST>(s, p, blk * tftq_col1_rows_per_wg(ST_D), tid);
         break;
-    case K_VECS: dequantize_small<T, POST>(s, p, blk, tid); break;
+    case K_VECS: dequantize_small<T, POST>(s, p, blk, tid, stage); break;
     default: break;
     }
 }

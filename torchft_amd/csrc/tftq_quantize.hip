@@ -398,57 +398,135 @@ DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 }
 
 // Short contiguous rows of whole 16-byte vectors (K_VECS, shape in tftq_device.h).
+// Scale of the row whose vectors a lane holds in v (maximum over the lanes of its team).
 template <typename T, int C>
-DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h)
+DEV float small_row_scale(const u32x4 (&v)[C], const SmallShape &h)
+{
+    float a = 0.0f;
+#pragma unroll
+    for (int k = 0; k < C; k++) {
+        a = fmaxf(a, vec_absmax<T>(v[k]));
+        // one vector after the other: with the 32 elements of four 16-bit vectors unpacked at
+        // once the kernel needs 81 registers instead of 70
+        if (C > 2) __builtin_amdgcn_sched_barrier(0);
+    }
+    if (h.lt >= 1) a = fmaxf(a, dpp_mov<0xB1>(a));   // quad_perm [1,0,3,2]
+    if (h.lt >= 2) a = fmaxf(a, dpp_mov<0x4E>(a));   // quad_perm [2,3,0,1]
+    if (h.lt >= 3) a = fmaxf(a, dpp_mov<0x141>(a));  // row_half_mirror
+    return calc_scale(a);
+}
+
+// Rows RBEG * teams .. REND * teams - 1 of the workgroup's rows (those up to `last`)
+// through the LDS stage: g0 is the address of the workgroup's first packed row.
+template <typename T, int C, int RBEG, int REND>
+DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)[8 / C][C], int row0, int last,
+                             uint8_t *g0, uint8_t *stage, int tid)
 {
     constexpr int EPV = Elem<T>::EPV;
-    constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane
     const int nvec = s.n / EPV;
-    const int row0 = blk * (h.teams * ROWS);
+    const int first = row0 + RBEG * h.teams;
+    if (first > last) return;  // same for the whole workgroup
+    uint8_t *gp = g0 + (int64_t)(RBEG * h.teams) * s.row_bytes;
+    const int mis = (int)((uintptr_t)gp & 127u);
+    const int len = (min(last, row0 + REND * h.teams - 1) - first + 1) * s.row_bytes;
+#pragma unroll
+    for (int r = RBEG; r < REND; r++) {
+        const int row = row0 + r * h.teams + h.t;
+        const float sc = small_row_scale<T, C>(v[r], h);
+        if (row > last) continue;
+        LDS_AS u32 *srow = (LDS_AS u32 *)(LDS_AS uint8_t *)(stage + mis + ((r - RBEG) * h.teams + h.t) * s.row_bytes);
+        if (row >= s.m) {  // padding row: zero (:93-95 on a zero-filled buffer)
+            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) srow[d] = 0;
+            continue;
+        }
+        if (h.l == 0) srow[0] = as_u(sc);
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            const int idx = k * h.team + h.l;
+            if (idx >= nvec) continue;
+            u32x4 x = v[r][k];
+            if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // unpacked anew, not kept from the maximum
+            const u32x2 o = vec_codes<T>(x, sc);
+            if constexpr (EPV == 4) srow[1 + idx] = o.x;
+            else *(LDS_AS u32x2_a4 *)(srow + 1 + 2 * idx) = o;
+        }
+    }
+    __syncthreads();
+    copy_out_span(stage, gp, len, tid);
+}
+
+// The rows of a workgroup are neighbours; when they lie in one slot their packed rows are
+// one span of bytes, which goes through LDS (copy_out_span) in two halves (rows of 8 to 64
+// 16-bit columns make up to 24 KB per workgroup, more than the stage holds).
+template <typename T, int C, bool STAGE>
+DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane: 8, 4 or 2
+    const int nvec = s.n / EPV;
+    const int nrows = h.teams * ROWS;
+    const int row0 = blk * nrows;
     const int m_pad = s.slice_rows * p.ws;
     const float inv = 1.0f / (float)s.slice_rows;
 
     u32x4 v[ROWS][C];
-    int row[ROWS];
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
-        row[r] = row0 + r * h.teams + h.t;
-        const int64_t e0 = (int64_t)min(row[r], s.m - 1) * s.row_stride;  // s.m >= 1: there are rows
+        const int row = row0 + r * h.teams + h.t;
+        const int64_t e0 = (int64_t)min(row, s.m - 1) * s.row_stride;  // s.m >= 1: there are rows
         GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + e0 * Elem<T>::ESZ);
 #pragma unroll
         for (int k = 0; k < C; k++) v[r][k] = LOAD_STREAM(in + min(k * h.team + h.l, nvec - 1));
     }
+    if constexpr (STAGE) {
+        // the workgroup's rows that exist, row0 .. last, and the slot of the first one
+        const int last = min(row0 + nrows, m_pad) - 1;
+        int slot0 = (int)((float)row0 * inv);
+        int j0 = row0 - slot0 * s.slice_rows;
+        if (j0 < 0) { --slot0; j0 += s.slice_rows; }
+        if (j0 >= s.slice_rows) { ++slot0; j0 -= s.slice_rows; }
+        if (j0 + (last - row0) < s.slice_rows) {  // one slot: one span.  Same for the whole workgroup
+            // the marker keeps the compiler from moving what this path and the one below have in
+            // common, the scales of all rows, in front of the branch (20 more registers)
+            asm volatile("; rows through the stage");
+            uint8_t *g0 = p.packed + (int64_t)slot0 * p.slot_size + s.slot_off + (int64_t)j0 * s.row_bytes;
+            quantize_small_span<T, C, 0, ROWS / 2>(s, h, v, row0, last, g0, stage, tid);
+            __syncthreads();  // the first half has been copied out of the stage
+            quantize_small_span<T, C, ROWS / 2, ROWS>(s, h, v, row0, last, g0, stage, tid);
+            return;
+        }
+    }
+    if constexpr (STAGE) asm volatile("; rows straight from the registers");
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
-        float a = 0.0f;
-#pragma unroll
-        for (int k = 0; k < C; k++) a = fmaxf(a, vec_absmax<T>(v[r][k]));
-        if (h.lt >= 1) a = fmaxf(a, dpp_mov<0xB1>(a));   // quad_perm [1,0,3,2]
-        if (h.lt >= 2) a = fmaxf(a, dpp_mov<0x4E>(a));   // quad_perm [2,3,0,1]
-        if (h.lt >= 3) a = fmaxf(a, dpp_mov<0x141>(a));  // row_half_mirror
-        if (row[r] >= m_pad) continue;
-        GLOBAL u32 *out = as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row[r], inv));
-        if (row[r] >= s.m) {
+        const int row = row0 + r * h.teams + h.t;
+        const float sc = small_row_scale<T, C>(v[r], h);
+        if (row >= m_pad) continue;
+        GLOBAL u32 *out = as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row, inv));
+        if (row >= s.m) {
             // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
             for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) out[d] = 0;
             continue;
         }
-        const float sc = calc_scale(a);
         if (h.l == 0) out[0] = as_u(sc);
 #pragma unroll
-        for (int k = 0; k < C; k++)
-            if (k * h.team + h.l < nvec) vec_quant_store<T>(v[r][k], sc, out + 1, k * h.team + h.l);
+        for (int k = 0; k < C; k++) {
+            u32x4 x = v[r][k];
+            if (STAGE && C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // as in quantize_small_span
+            if (k * h.team + h.l < nvec) vec_quant_store<T>(x, sc, out + 1, k * h.team + h.l);
+        }
     }
 }
 
-template <typename T>
-DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid)
+// STAGE: the kernel has the LDS stage (the wide variant does not)
+template <typename T, bool STAGE>
+DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
     const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
-    if (h.c == 1) quantize_small_c<T, 1>(s, p, blk, tid, h);
-    else if (h.c == 2) quantize_small_c<T, 2>(s, p, blk, tid, h);
-    else if (h.c == 3) quantize_small_c<T, 3>(s, p, blk, tid, h);
-    else quantize_small_c<T, 4>(s, p, blk, tid, h);
+    if (h.c == 1) quantize_small_c<T, 1, STAGE>(s, p, blk, tid, h, stage);
+    else if (h.c == 2) quantize_small_c<T, 2, STAGE>(s, p, blk, tid, h, stage);
+    else if (h.c == 3) quantize_small_c<T, 3, STAGE>(s, p, blk, tid, h, stage);
+    else quantize_small_c<T, 4, STAGE>(s, p, blk, tid, h, stage);
 }
 
 template <typename T, bool INLINE, bool WIDE>
@@ -476,7 +554,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
     case K_GEN8: quantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: quantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
     case K_COL1: quantize_col1<T>(s, p, blk * tftq_col1_rows_per_wg(ST_Q), tid); break;
-    case K_VECS: quantize_small<T>(s, p, blk, tid); break;
+    case K_VECS: quantize_small<T, !WIDE>(s, p, blk, tid, stage); break;
     default: break;
     }
 }
