@@ -44,6 +44,8 @@ DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
 }
 
 constexpr int Q_STAGE_BYTES = 16640;  // 8 rows of 2052 bytes (2048 16-bit columns) + 127 bytes of offset, rounded up (see copy_out_span)
+// the wide kernel, whose three workgroups per CU leave each 53 KB of LDS: one row of 32768 16-bit columns
+constexpr int Q_STAGE_BYTES_WIDE = 32912;
 
 // Contiguous, 16-byte aligned rows of at most TEAM * KMAX vectors.  The KMAX
 // loads of a lane are issued back to back without a branch in between: lanes
@@ -255,19 +257,22 @@ DEV void quantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, flo
     const int r0 = blk * R;
     const int team = TEAM == 64 ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid / TEAM;
     const int lane = tid & (TEAM - 1);
-    if constexpr (!WIDE) {
+    {
+        constexpr int KMAX = WIDE && TEAM == 256 ? 2 * QV : QV;  // vectors per lane that the kernel keeps in registers
+        constexpr int STAGE_BYTES = WIDE ? Q_STAGE_BYTES_WIDE : Q_STAGE_BYTES;
         const int nvec = s.n / Elem<T>::EPV;
         const int last = r0 + R - 1;
-        if (last < s.m && nvec <= QV * TEAM) {
+        if (last < s.m && nvec <= KMAX * TEAM) {
             const int slot = r0 / s.slice_rows;
             const int j = r0 - slot * s.slice_rows;
             uint8_t *g0 = p.packed + (int64_t)slot * p.slot_size + s.slot_off + (int64_t)j * s.row_bytes;
             const int mis = (int)((uintptr_t)g0 & 127u);
             const int len = R * s.row_bytes;
-            if (j + R <= s.slice_rows && mis + len <= Q_STAGE_BYTES) {  // same for the whole workgroup
+            if (j + R <= s.slice_rows && mis + len <= STAGE_BYTES) {  // same for the whole workgroup
                 LDS_AS u32 *srow = (LDS_AS u32 *)(LDS_AS uint8_t *)(stage + mis + team * s.row_bytes);
                 if (nvec <= (QV / 2) * TEAM) quantize_vec_k<T, TEAM, QV / 2, true>(s, p, r0 + team, lane, lds, srow);
-                else quantize_vec_k<T, TEAM, QV, true>(s, p, r0 + team, lane, lds, srow);
+                else if (KMAX == QV || nvec <= QV * TEAM) quantize_vec_k<T, TEAM, QV, true>(s, p, r0 + team, lane, lds, srow);
+                else quantize_vec_k<T, TEAM, KMAX, true>(s, p, r0 + team, lane, lds, srow);
                 __syncthreads();
                 copy_out_span(stage, g0, len, tid);
                 return;
@@ -458,7 +463,7 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
 // The rows of a workgroup are neighbours; when they lie in one slot their packed rows are
 // one span of bytes, which goes through LDS (copy_out_span) in two halves (rows of 8 to 64
 // 16-bit columns make up to 24 KB per workgroup, more than the stage holds).
-template <typename T, int C, bool STAGE>
+template <typename T, int C>
 DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
     constexpr int EPV = Elem<T>::EPV;
@@ -478,7 +483,7 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
 #pragma unroll
         for (int k = 0; k < C; k++) v[r][k] = LOAD_STREAM(in + min(k * h.team + h.l, nvec - 1));
     }
-    if constexpr (STAGE) {
+    {
         // the workgroup's rows that exist, row0 .. last, and the slot of the first one
         const int last = min(row0 + nrows, m_pad) - 1;
         int slot0 = (int)((float)row0 * inv);
@@ -496,7 +501,7 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
             return;
         }
     }
-    if constexpr (STAGE) asm volatile("; rows straight from the registers");
+    asm volatile("; rows straight from the registers");
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
         const int row = row0 + r * h.teams + h.t;
@@ -512,31 +517,32 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
 #pragma unroll
         for (int k = 0; k < C; k++) {
             u32x4 x = v[r][k];
-            if (STAGE && C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // as in quantize_small_span
+            if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // as in quantize_small_span
             if (k * h.team + h.l < nvec) vec_quant_store<T>(x, sc, out + 1, k * h.team + h.l);
         }
     }
 }
 
-// STAGE: the kernel has the LDS stage (the wide variant does not)
-template <typename T, bool STAGE>
+template <typename T>
 DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
     const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
-    if (h.c == 1) quantize_small_c<T, 1, STAGE>(s, p, blk, tid, h, stage);
-    else if (h.c == 2) quantize_small_c<T, 2, STAGE>(s, p, blk, tid, h, stage);
-    else if (h.c == 3) quantize_small_c<T, 3, STAGE>(s, p, blk, tid, h, stage);
-    else quantize_small_c<T, 4, STAGE>(s, p, blk, tid, h, stage);
+    if (h.c == 1) quantize_small_c<T, 1>(s, p, blk, tid, h, stage);
+    else if (h.c == 2) quantize_small_c<T, 2>(s, p, blk, tid, h, stage);
+    else if (h.c == 3) quantize_small_c<T, 3>(s, p, blk, tid, h, stage);
+    else quantize_small_c<T, 4>(s, p, blk, tid, h, stage);
 }
 
 template <typename T, bool INLINE, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[4];
-    __shared__ __align__(16) uint8_t stage[WIDE ? 16 : Q_STAGE_BYTES];  // see copy_out_span
-    // 60 KB of dynamic LDS, asked for at the launch only when the plan has rows that need it
-    // (it limits a CU to two workgroups)
+    __shared__ __align__(16) uint8_t stage_regular[WIDE ? 16 : Q_STAGE_BYTES];  // see copy_out_span
+    // Dynamic LDS of the wide kernel: Q_STAGE_BYTES_WIDE as its stage, or 60 KB when the plan has
+    // rows that are parked there (which limits a CU to two workgroups); a workgroup uses it
+    // for one or the other.
     extern __shared__ u32x4 park[];
+    uint8_t *stage = WIDE ? (uint8_t *)park : stage_regular;
     Seg s;
     int vb;
     if (!locate<INLINE, ST_Q>(p, inl, s, vb)) return;
@@ -554,7 +560,7 @@ __global__ __launch_bounds__(TFTQ_WG) void k_quantize(const KParams p, const Inl
     case K_GEN8: quantize_gen<T, 8>(s, p, blk * 32 + (tid >> 3), tid & 7); break;
     case K_GEN1: quantize_gen<T, 1>(s, p, blk * 256 + tid, 0); break;
     case K_COL1: quantize_col1<T>(s, p, blk * tftq_col1_rows_per_wg(ST_Q), tid); break;
-    case K_VECS: quantize_small<T, !WIDE>(s, p, blk, tid, stage); break;
+    case K_VECS: quantize_small<T>(s, p, blk, tid, stage); break;
     default: break;
     }
 }
@@ -565,7 +571,8 @@ static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, 
 {
     const unsigned grid = grid_of(kp);
     if (wide) {
-        const unsigned lds = parked ? TFTQ_Q_PARKED * TFTQ_WG * 16u : 0u;
+        const unsigned lds = parked ? TFTQ_Q_PARKED * TFTQ_WG * 16u : (unsigned)Q_STAGE_BYTES_WIDE;
+        static_assert(TFTQ_Q_PARKED * TFTQ_WG * 16 >= Q_STAGE_BYTES_WIDE, "the parking area also serves as the stage");
         if (use_inline) return launch_kernel(k_quantize<T, true, true>, grid, lds, st, kp, inl);
         return launch_kernel(k_quantize<T, false, true>, grid, lds, st, kp, inl);
     }
