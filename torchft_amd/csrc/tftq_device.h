@@ -211,7 +211,8 @@ template <> struct Elem<float> {
     DEV static float load(uint64_t base, int64_t idx) { return as_global<const float>(base)[idx]; }
     DEV static void store(uint64_t base, int64_t idx, float v) { as_global<float>(base)[idx] = v; }
     DEV static float rounded(float v) { return v; }  // v as a stored element reads back
-    // elements idx and idx + 1 with one access
+    // elements idx and idx + 1 with one access (streaming: neighbouring lanes take neighbouring
+    // pairs, so a wavefront covers whole lines)
     DEV static void load2(uint64_t base, int64_t idx, float &a, float &b)
     {
         const u32x2 w = LOAD_STREAM((GLOBAL const u32x2_a4 *)(as_global<const float>(base) + idx));
@@ -221,7 +222,7 @@ template <> struct Elem<float> {
     DEV static void store2(uint64_t base, int64_t idx, float a, float b)
     {
         const u32x2 w = {as_u(a), as_u(b)};
-        *(GLOBAL u32x2_a4 *)(as_global<float>(base) + idx) = w;
+        STORE_STREAM(w, (GLOBAL u32x2_a4 *)(as_global<float>(base) + idx));
     }
 };
 
@@ -263,7 +264,7 @@ template <> struct Elem<bf16_tag> {
     }
     DEV static void store2(uint64_t base, int64_t idx, float a, float b)
     {
-        *(GLOBAL u32_a2 *)(as_global<uint16_t>(base) + idx) = pack2(a, b);
+        STORE_STREAM(pack2(a, b), (GLOBAL u32_a2 *)(as_global<uint16_t>(base) + idx));
     }
 };
 
@@ -316,7 +317,7 @@ template <> struct Elem<f16_tag> {
     }
     DEV static void store2(uint64_t base, int64_t idx, float a, float b)
     {
-        *(GLOBAL u32_a2 *)(as_global<uint16_t>(base) + idx) = pack2(a, b);
+        STORE_STREAM(pack2(a, b), (GLOBAL u32_a2 *)(as_global<uint16_t>(base) + idx));
     }
 };
 

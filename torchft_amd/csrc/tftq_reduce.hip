@@ -752,7 +752,8 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
             u32x2 o;
             o.x = as_u(s2);
             o.y = pack_fp8x4(scale_div<GDIV, IEEE>(acc[k], s2, p), 0.0f, 0.0f, 0.0f) & 0xFFu;
-            *(GLOBAL u32x2_a4 *)as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off[k]) = o;
+            // streaming: neighbouring lanes write neighbouring rows, whole lines per wavefront
+            STORE_STREAM(o, (GLOBAL u32x2_a4 *)as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off[k]));
         }
     }
 }
