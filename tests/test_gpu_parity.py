@@ -273,6 +273,10 @@ def test_dequantize_rows_through_lds_spans(q, oracle, dtype):
         n = row_bytes // esz
         for m, off in ((37, 0), (9, 2 * (4 // esz)), (70, 30 * (4 // esz) + 64), (3, 1)):
             cases.append((m, n, off))
+    # rows of 1 to 31 whole vectors: several rows per lane, a workgroup's rows in two halves
+    for row_bytes, m in ((16, 5000), (48, 3), (48, 2500), (80, 1500), (144, 700), (272, 300), (400, 333), (496, 130)):
+        for off in (0, 4 // esz, 25 * (4 // esz), 1):
+            cases.append((m, row_bytes // esz, off))
     cpu_src = []
     for m, n, _ in cases:
         t = torch.randn(m, n, generator=g) * 0.3
@@ -280,6 +284,8 @@ def test_dequantize_rows_through_lds_spans(q, oracle, dtype):
         if dtype == torch.float16:
             t[m // 2] = 0.0
             t[m // 2, 0] = 6e-8
+        if n < 16:
+            t[0] = 0.0  # an all-zero row
         cpu_src.append(t.to(dtype))
     for ws in (1, 4):
         b = oracle.fused_quantize_into_fp8(list(cpu_src), ws)
