@@ -206,6 +206,10 @@ def run_ceilings(args) -> int:
               7, rows, 1, NT, PLAIN),
              ("reduce's accesses, rows in workgroup order", 7, rows, 0, NT, PLAIN),
              ("reduce's accesses, an eighth per XCD, wavefronts start on 128-byte lines", 8, rows, 1, NT, PLAIN),
+             ("quantize's accesses: 8 KB rows -> 4100-byte packed rows through LDS, rows in workgroup order",
+              10, 8 * rows, 0, NT, NT),
+             ("quantize's accesses, packed rows straight from the registers (plain stores)",
+              10, 8 * rows, 0, NT, PLAIN),
              ("dequantize's accesses: 4100-byte packed rows -> 8 KB rows, rows in workgroup order",
               9, 8 * rows, 0, NT, NT),
              ("dequantize's accesses, an eighth of the rows per XCD", 9, 8 * rows, 1, NT, NT)]

@@ -27,6 +27,11 @@
 //            what it costs that packed rows start anywhere
 //   DEQ      dequantize on 16-bit rows of 4096 columns: one wavefront per row, a lane loads
 //            8 x 8 bytes of the packed row and stores 8 x 16 bytes of the 8 KB tensor row
+//   QNT      quantize on 16-bit rows of 4096 columns: four rows per workgroup, one wavefront per
+//            row, a lane loads 8 x 16 bytes of the 8 KB tensor row and produces 8 x 8 bytes of
+//            the packed row of row_bytes.  nt_stores: the workgroup assembles its four packed
+//            rows in LDS and writes them as whole lines with streaming stores, as the product
+//            does; otherwise plain 8-byte stores straight from the registers.  Rows of one slot.
 //
 // `eighths` (patterns only): workgroup ids go round-robin to the 8 XCDs of the chip; with
 // eighths XCD x works through the x-th contiguous eighth of the rows, without it workgroup
@@ -43,7 +48,7 @@ typedef u32x2 u32x2_a4 __attribute__((aligned(4)));
 #define GLOBAL __attribute__((address_space(1)))
 
 enum { C_RO = 0, C_WO = 1, C_R2W1 = 2, C_R1W2 = 3, C_R4W1 = 4, C_R1W4 = 5, C_R8W1 = 6,
-       C_RED = 7, C_RED_LINE = 8, C_DEQ = 9, C_KINDS = 10 };
+       C_RED = 7, C_RED_LINE = 8, C_DEQ = 9, C_QNT = 10, C_KINDS = 11 };
 
 template <typename V, bool NT>
 __device__ __forceinline__ V ld(GLOBAL const V *p)
@@ -172,6 +177,55 @@ __global__ __launch_bounds__(256) void k_dequantize_pattern(const uint8_t *packe
     }
 }
 
+template <bool NTL, bool STAGED>
+__global__ __launch_bounds__(256) void k_quantize_pattern(const uint8_t *tensor, uint8_t *packed, int rows,
+                                                          int row_bytes, int per_xcd)
+{
+    __shared__ __align__(16) uint8_t stage[16640];
+    const int r0 = piece_of(per_xcd) * 4;
+    if (r0 >= rows) return;  // rows is a multiple of 4
+    const int t = threadIdx.x, wave = t >> 6, l = t & 63;
+    GLOBAL const u32x4 *in = (GLOBAL const u32x4 *)(uint64_t)(tensor + (int64_t)(r0 + wave) * 8192);
+    u32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = NTL ? __builtin_nontemporal_load(in + k * 64 + l) : in[k * 64 + l];
+    uint8_t *g0 = packed + (int64_t)r0 * row_bytes;
+    if (STAGED) {
+        const int mis = (int)((uint64_t)g0 & 127u);
+        typedef __attribute__((address_space(3))) uint8_t lds_u8;
+        lds_u8 *srow = (lds_u8 *)stage + mis + wave * row_bytes;
+        if (l == 0) *(__attribute__((address_space(3))) u32 *)srow = v[0].x;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const u32x2 o = {v[k].x ^ v[k].z, v[k].y ^ v[k].w};
+            *(__attribute__((address_space(3))) u32x2_a4 *)(srow + 4 + 8 * (k * 64 + l)) = o;
+        }
+        __syncthreads();
+        const int end = mis + 4 * row_bytes;
+        GLOBAL uint8_t *line0 = (GLOBAL uint8_t *)(uint64_t)(g0 - mis);
+        for (int c = t; c < (end + 15) >> 4; c += 256) {
+            const int lo = 16 * c;
+            const u32x4 x = *(const __attribute__((address_space(3))) u32x4 *)((lds_u8 *)stage + lo);
+            if (lo >= mis && lo + 16 <= end) {
+                __builtin_nontemporal_store(x, (GLOBAL u32x4 *)(line0 + lo));
+            } else {
+                const u32 w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    if (lo + 4 * d >= mis && lo + 4 * d < end) *(GLOBAL u32 *)(line0 + lo + 4 * d) = w[d];
+            }
+        }
+    } else {
+        GLOBAL u32 *out = (GLOBAL u32 *)(uint64_t)(g0 + (int64_t)wave * row_bytes);
+        if (l == 0) out[0] = v[0].x;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const u32x2 o = {v[k].x ^ v[k].z, v[k].y ^ v[k].w};
+            *(GLOBAL u32x2_a4 *)(out + 1 + 2 * (k * 64 + l)) = o;
+        }
+    }
+}
+
 // Bytes that one launch of `kind` reads and writes; units = workgroups of the plain mixes, rows
 // of the patterns.
 extern "C" int tftq_ceiling_bytes(int kind, int64_t units, int row_bytes, int64_t *read_bytes, int64_t *write_bytes)
@@ -181,6 +235,9 @@ extern "C" int tftq_ceiling_bytes(int kind, int64_t units, int row_bytes, int64_
     if (kind == C_DEQ) {
         *read_bytes = units * (int64_t)row_bytes;
         *write_bytes = units * 8192;
+    } else if (kind == C_QNT) {
+        *read_bytes = units * 8192;
+        *write_bytes = units * (int64_t)row_bytes;
     } else if (kind == C_RED || kind == C_RED_LINE) {
         *read_bytes = units * (int64_t)row_bytes * 8;
         *write_bytes = units * (int64_t)row_bytes;
@@ -194,7 +251,8 @@ extern "C" int tftq_ceiling_bytes(int kind, int64_t units, int row_bytes, int64_
 // One launch on `stream`.  Plain mixes: src and dst hold what tftq_ceiling_bytes says.  RED,
 // RED_LINE: dst is the buffer of 8 slots of slot_size bytes, updated in place (RED_LINE: slot_size
 // a multiple of 128), src is not used, 20 <= row_bytes <= 4100.  DEQ: src holds the packed rows
-// (row_bytes >= 4100 apart), dst the rows of 8192 bytes.  nt_loads / nt_stores pick streaming
+// (row_bytes >= 4100 apart), dst the rows of 8192 bytes.  QNT: src holds rows of 8192 bytes, dst
+// the packed rows (row_bytes = 4100, units a multiple of 4).  nt_loads / nt_stores pick streaming
 // (nontemporal) accesses; the patterns store as the product does (RED plain, DEQ per nt_stores).
 // Returns 0, a hipError_t, or -1 for bad arguments.
 extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t units, int64_t slot_size,
@@ -248,6 +306,18 @@ extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t
         else if (nt_loads) hipLaunchKernelGGL((k_dequantize_pattern<true, false>), g, block, 0, s, a, b, rows, row_bytes, px);
         else if (nt_stores) hipLaunchKernelGGL((k_dequantize_pattern<false, true>), g, block, 0, s, a, b, rows, row_bytes, px);
         else hipLaunchKernelGGL((k_dequantize_pattern<false, false>), g, block, 0, s, a, b, rows, row_bytes, px);
+        break;
+    }
+    case C_QNT: {
+        if (row_bytes != 4100 || (units & 3)) return -1;
+        const int wgs = (int)(units / 4);
+        const int px = eighths ? (wgs + 7) / 8 : 0;
+        const dim3 g(eighths ? (unsigned)(8 * px) : (unsigned)wgs);
+        const int rows = (int)units;
+        if (nt_loads && nt_stores) hipLaunchKernelGGL((k_quantize_pattern<true, true>), g, block, 0, s, a, b, rows, row_bytes, px);
+        else if (nt_loads) hipLaunchKernelGGL((k_quantize_pattern<true, false>), g, block, 0, s, a, b, rows, row_bytes, px);
+        else if (nt_stores) hipLaunchKernelGGL((k_quantize_pattern<false, true>), g, block, 0, s, a, b, rows, row_bytes, px);
+        else hipLaunchKernelGGL((k_quantize_pattern<false, false>), g, block, 0, s, a, b, rows, row_bytes, px);
         break;
     }
     default: return -1;
