@@ -431,9 +431,9 @@ def main() -> int:
         step(i)
     torch.cuda.synchronize()
 
-    # Which stage takes longest: three untimed steps with events around every stage.
-    probe_events = [[ev() for _ in range(4)] for _ in range(3)]
-    for i in range(3):
+    # Which stage takes longest: eight untimed steps with events around every stage.
+    probe_events = [[ev() for _ in range(4)] for _ in range(8)]
+    for i in range(8):
         step(i, probe_events[i])
     torch.cuda.synchronize()
     probe_ms = stage_means(probe_events, range(3))
@@ -442,15 +442,20 @@ def main() -> int:
 
     # The timed region: K steps, events only around the dominant kernel (every event record
     # costs ~3 us of dispatch gap: 4 records per step made the step 12 us longer).
+    # The pair is recorded on every fourth step: a pair costs the step about 5 us.
+    stride = 4 if args.steps >= 8 else 1
     all_events = [[ev() for _ in range(4)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i, all_events[i], only=dom)
+        if i % stride == 0:
+            step(i, all_events[i], only=dom)
+        else:
+            step(i)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    dominant_ms = stage_means(all_events, [dom])[dominant]
+    dominant_ms = stage_means(all_events[::stride], [dom])[dominant]
 
     # What a pair of event records reads with no kernel between them, on a busy stream: the
     # part of every event-bracketed duration that is not the kernel.
@@ -532,8 +537,8 @@ def main() -> int:
                 "us_between_events": round(dominant_ms * 1e3, 2),
                 "event_pair_us": round(event_pair_ms * 1e3, 2),
                 "frac_without_correction": round(ab[dominant] / (dominant_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                "timing": "HIP events around the kernel inside the timed quantize -> reduce -> dequantize "
-                          "steps (us_between_events), less event_pair_us, what two records with nothing "
+                "timing": "HIP events around the kernel on every fourth of the timed quantize -> reduce -> "
+                          "dequantize steps (us_between_events), less event_pair_us, what two records with nothing "
                           "between them read on the same stream",
                 "alone": stages_alone[dominant],
                 "traffic": profiled_traffic.get(dominant),
