@@ -3,7 +3,8 @@
 // For random tensor lists this program builds plans with the library's own
 // planner (tftq_plan.cpp, linked in), walks every workgroup id of the launch
 // grid through a host restatement of the kernels' lookup (inline tables: the
-// per-XCD dealt rows; device tables: chunk dealing, bucket map, binary search)
+// per-XCD dealt rows; device tables: chunk dealing, bucket map, binary search,
+// and for reduce the quarters of workgroups that its wavefronts take one each)
 // and checks that every block of every tensor is visited exactly once, in all
 // three stages.  Prints "ok <plans> plans" on success.
 
@@ -42,12 +43,17 @@ static bool locate_inline(const tftq_plan *p, int st, uint32_t b, int *seg, int 
     return true;
 }
 
-static bool locate_table(const tftq_plan *p, int st, uint32_t b, int *seg, int *vb, size_t *max_steps)
+// wave: the wavefront of the workgroup (stages that number quarters of workgroups: reduce)
+static bool locate_table(const tftq_plan *p, int st, uint32_t b, int wave, int *seg, int *vb, size_t *max_steps)
 {
     const int x = (int)(b & 7), i = (int)(b >> 3);
     const int cs = p->index[st].chunk_shift;
-    const int v = ((((i >> cs) << 3) + x) << cs) + (i & ((1 << cs) - 1));
+    int v = ((((i >> cs) << 3) + x) << cs) + (i & ((1 << cs) - 1));
     if (v >= p->nwg[st]) return false;
+    if (p->index[st].pieces) {
+        v = 4 * v + wave;
+        if (v >= p->index[st].pieces) return false;
+    }
     const uint8_t *tab = p->blob.data();
     const size_t map_idx = (size_t)(v >> p->index[st].shift);
     const size_t map_bytes = (size_t)p->index[st].map_off + (map_idx + 2) * sizeof(MapEnt);
@@ -100,7 +106,12 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
         }
     }
     for (int st = 0; st < 3; st++) {
-        // blocks each segment must receive
+        // blocks each segment must receive: workgroups, or quarters of workgroups (pieces)
+        const bool pieces = !inl && p->index[st].pieces > 0;
+        if (pieces != (!inl && st == ST_R)) {
+            printf("stage %d: pieces %d\n", st, (int)pieces);
+            return 1;
+        }
         std::vector<std::vector<uint8_t>> seen((size_t)n);
         int64_t total = 0;
         for (int i = 0; i < n; i++) {
@@ -108,40 +119,68 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
             const int64_t m_pad = (int64_t)s.slice_rows * ws;
             const int64_t rows = st == ST_Q ? m_pad : st == ST_R ? s.slice_rows : s.m;
             const int per_wg = tftq_rows_per_wg(s, st, dtype == TFTQ_F32 ? 4 : 2, ws);
-            const int64_t blocks = (rows + per_wg - 1) / per_wg;
+            int64_t blocks = (rows + per_wg - 1) / per_wg;
+            if (pieces) {
+                blocks = tftq_reduce_pieces(s, dtype == TFTQ_F32 ? 4 : 2, ws, blocks);
+                // every row of the tensor lies in one of its pieces
+                const bool whole = s.kind[st] == K_GEN256 || s.kind[st] == K_COL1;
+                if (whole ? blocks * per_wg < 4 * rows : blocks * (per_wg / 4) < rows || (blocks - 1) * (per_wg / 4) >= rows + (rows == 0)) {
+                    printf("stage %d segment %d: %lld pieces for %lld rows\n", st, i, (long long)blocks, (long long)rows);
+                    return 1;
+                }
+                if (tftq_reduce_kind_has_barriers(s.kind[st]) && (s.wg_begin[st] & 3)) {
+                    printf("stage %d segment %d: a kind with barriers starts at piece %d\n", st, i, s.wg_begin[st]);
+                    return 1;
+                }
+            }
             seen[(size_t)i].assign((size_t)blocks, 0);
             total += blocks;
         }
-        if (total != p->nwg[st]) {
+        const int64_t launched = pieces ? 4 * (int64_t)p->nwg[st] : p->nwg[st];
+        if (pieces ? (total > p->index[st].pieces || p->index[st].pieces > launched || launched > p->index[st].pieces + 3)
+                   : total != p->nwg[st]) {
             printf("stage %d: %lld blocks but nwg %d\n", st, (long long)total, p->nwg[st]);
             return 1;
         }
         const int64_t per_xcd = inl ? p->dealt_per_xcd[st] : p->index[st].per_xcd;
         const int64_t grid = 8 * per_xcd;
-        const int64_t slack = inl ? 8 * n : ((int64_t)8 << p->index[st].chunk_shift) + total / 32;
-        if (grid < total || grid > total + slack) {
-            printf("stage %d: grid %lld for %lld workgroups\n", st, (long long)grid, (long long)total);
+        const int64_t wgs_needed = p->nwg[st];
+        const int64_t slack = inl ? 8 * n : ((int64_t)8 << p->index[st].chunk_shift) + wgs_needed / 32;
+        if (grid < wgs_needed || grid > wgs_needed + slack) {
+            printf("stage %d: grid %lld for %lld workgroups\n", st, (long long)grid, (long long)wgs_needed);
             return 1;
         }
         int64_t visited = 0;
         size_t max_steps = 0;
         for (int64_t b = 0; b < grid; b++) {
-            int sg = -1, vb = -1;
-            const bool ok = inl ? locate_inline(p, st, (uint32_t)b, &sg, &vb)
-                                : locate_table(p, st, (uint32_t)b, &sg, &vb, &max_steps);
-            if (!ok) continue;
-            if (sg < 0 || sg >= n) {
-                printf("stage %d id %lld: segment %d\n", st, (long long)b, sg);
-                return 1;
+            for (int wave = 0; wave < (pieces ? 4 : 1); wave++) {
+                int sg = -1, vb = -1;
+                const bool ok = inl ? locate_inline(p, st, (uint32_t)b, &sg, &vb)
+                                    : locate_table(p, st, (uint32_t)b, wave, &sg, &vb, &max_steps);
+                if (!ok) continue;
+                if (sg < 0 || sg >= n) {
+                    printf("stage %d id %lld: segment %d\n", st, (long long)b, sg);
+                    return 1;
+                }
+                const int64_t blk = (int64_t)vb - p->segs[(size_t)sg].wg_begin[st];
+                if (pieces && blk >= (int64_t)seen[(size_t)sg].size()) {
+                    // padding in front of a tensor whose kind needs whole workgroups: it must
+                    // fall to a kind whose wavefronts simply find no row
+                    if (blk >= 0 && !tftq_reduce_kind_has_barriers(p->segs[(size_t)sg].kind[st]) && blk < (int64_t)seen[(size_t)sg].size() + 3)
+                        continue;
+                }
+                if (blk < 0 || blk >= (int64_t)seen[(size_t)sg].size() || seen[(size_t)sg][(size_t)blk]) {
+                    printf("stage %d id %lld: segment %d block %lld out of range or visited twice\n", st,
+                           (long long)b, sg, (long long)blk);
+                    return 1;
+                }
+                if (pieces && tftq_reduce_kind_has_barriers(p->segs[(size_t)sg].kind[st]) && (blk & 3) != wave) {
+                    printf("stage %d id %lld: a workgroup of a kind with barriers is split\n", st, (long long)b);
+                    return 1;
+                }
+                seen[(size_t)sg][(size_t)blk] = 1;
+                visited++;
             }
-            const int64_t blk = (int64_t)vb - p->segs[(size_t)sg].wg_begin[st];
-            if (blk < 0 || blk >= (int64_t)seen[(size_t)sg].size() || seen[(size_t)sg][(size_t)blk]) {
-                printf("stage %d id %lld: segment %d block %lld out of range or visited twice\n", st,
-                       (long long)b, sg, (long long)blk);
-                return 1;
-            }
-            seen[(size_t)sg][(size_t)blk] = 1;
-            visited++;
         }
         if (visited != total) {
             printf("stage %d: visited %lld of %lld\n", st, (long long)visited, (long long)total);

@@ -382,11 +382,15 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
     } else {
         // everything the first steps need from the kernel arguments in one round of scalar loads
         asm volatile("" ::"s"(p.table), "s"(p.ptrs), "s"(p.map_off), "s"(p.sorted_off), "s"(p.map_shift), "s"(p.chunk_shift),
-                     "s"(p.nwg), "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
+                     "s"(p.nwg), "s"(p.pieces), "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
         // chunks of 2^chunk_shift consecutive workgroups go to the XCDs in turn
         const int cs = p.chunk_shift;
         vb = ((((i >> cs) << 3) + x) << cs) + (i & ((1 << cs) - 1));
         if (vb >= p.nwg) return false;
+        if (STAGE == ST_R && p.pieces) {  // this wavefront's quarter of the workgroup (tftq_reduce_pieces)
+            vb = 4 * vb + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+            if (vb >= p.pieces) return false;
+        }
         const uint64_t tab = (uint64_t)p.table;
         typedef int32_t MapPair __attribute__((ext_vector_type(4), aligned(8)));
         const MapPair m = *(const CONSTANT MapPair *)(tab + (uint64_t)p.map_off +
@@ -490,11 +494,13 @@ static inline void work_mapping(const tftq_plan *plan, int stage, KParams *kp)
         kp->dealt = plan->dealt[stage];
         kp->per_xcd = plan->dealt_per_xcd[stage];
         kp->natural = plan->natural[stage] ? 1 : 0;
+        kp->pieces = 0;
         kp->map_shift = kp->chunk_shift = 0;
         kp->sorted_off = kp->map_off = 0;
     } else {
         kp->per_xcd = plan->index[stage].per_xcd;
         kp->natural = 0;
+        kp->pieces = plan->index[stage].pieces;
         kp->map_shift = plan->index[stage].shift;
         kp->chunk_shift = plan->index[stage].chunk_shift;
         kp->sorted_off = plan->index[stage].sorted_off;

@@ -149,6 +149,24 @@ static inline int tftq_rows_per_wg(const Seg &s, int st, int esz, int ws)
     return teams;
 }
 
+// Reduce on long lists (device table) numbers its work in quarters of workgroups, one
+// wavefront each, because most tensors of such lists have a row or two per slot and a
+// workgroup per tensor would be three quarters idle: wavefront w of workgroup v takes piece
+// 4 v + w, finds its tensor itself, and acts as wavefront (piece - first piece) % 4 of
+// workgroup (piece - first piece) / 4 of that tensor.  The kinds whose teams are wavefronts
+// or less need as many pieces as have rows; the 256-lane kind, whose wavefronts meet at
+// barriers, and rows of one column (rows dealt across the whole workgroup) take four pieces
+// per workgroup, the former starting at a multiple of four.
+static inline bool tftq_reduce_kind_has_barriers(uint8_t kind) { return kind == K_GEN256; }
+static inline int64_t tftq_reduce_pieces(const Seg &s, int esz, int ws, int64_t wgs)
+{
+    if (wgs == 0) return 0;
+    if (s.kind[ST_R] == K_GEN256 || s.kind[ST_R] == K_COL1) return 4 * wgs;
+    const int per_piece = tftq_rows_per_wg(s, ST_R, esz, ws) / 4;
+    return ((int64_t)s.slice_rows + per_piece - 1) / per_piece;
+}
+
+
 struct InlineTable {
     Seg s[TFTQ_N_INLINE];
 };
@@ -183,6 +201,7 @@ struct TableIndex {
     int32_t shift;
     int32_t chunk_shift;
     int32_t per_xcd;     // workgroup ids per XCD in the grid
+    int32_t pieces;      // reduce: the work is numbered in quarters of workgroups (see tftq_reduce_pieces); else 0
 };
 
 struct tftq_plan {
@@ -216,6 +235,7 @@ struct KParams {
     int32_t rank;
     int32_t per_xcd;    // workgroup ids per XCD in the grid
     int32_t natural;    // inline table only: workgroup id b is piece b of the work, not piece b / 8 of XCD b % 8
+    int32_t pieces;     // device table, reduce: number of quarter-workgroup pieces (0: whole workgroups)
     int32_t map_shift;  // device table only, as are the next three
     int32_t chunk_shift;
     int64_t sorted_off;

@@ -220,14 +220,22 @@ static int build_table(tftq_plan *p, const int32_t (*wgs)[3])
         std::vector<int32_t> ord;
         work_order(p, st, ord);
         sorted[st].resize(nseg);
-        int32_t begin = 0;
-        for (size_t k = 0; k < nseg; k++) {  // workgroup numbers in sorted order
+        // Reduce numbers quarters of workgroups (tftq_reduce_pieces), the others whole workgroups.
+        const bool pieces = st == ST_R;
+        int64_t begin = 0;
+        for (size_t k = 0; k < nseg; k++) {  // workgroup (piece) numbers in sorted order
             const int32_t i = ord[k];
-            p->segs[(size_t)i].wg_begin[st] = begin;
-            sorted[st][k] = SortEnt{begin, i};
-            begin += wgs[i][st];
+            const Seg &sg = p->segs[(size_t)i];
+            if (pieces && tftq_reduce_kind_has_barriers(sg.kind[st])) begin = (begin + 3) & ~(int64_t)3;
+            if (begin > INT32_MAX - 4096) return TFTQ_E_SHAPE;
+            p->segs[(size_t)i].wg_begin[st] = (int32_t)begin;
+            sorted[st][k] = SortEnt{(int32_t)begin, i};
+            begin += pieces ? tftq_reduce_pieces(sg, p->esz, p->ws, wgs[i][st]) : wgs[i][st];
         }
-        const int64_t nwg = p->nwg[st];
+        if (begin > INT32_MAX - 4096) return TFTQ_E_SHAPE;
+        p->index[st].pieces = pieces ? (int32_t)begin : 0;
+        if (pieces) p->nwg[st] = (int32_t)((begin + 3) / 4);
+        const int64_t nwg = begin;  // what the map is indexed by
         int shift = 0;
         while ((nwg >> shift) > 4 * (int64_t)nseg) shift++;
         const int64_t nb = (nwg >> shift) + 1;  // buckets; map[] has one more entry
@@ -243,10 +251,11 @@ static int build_table(tftq_plan *p, const int32_t (*wgs)[3])
             map[st][(size_t)b] = MapEnt{(int32_t)k, sorted[st][k].seg};
         }
         p->index[st].shift = shift;
+        const int64_t nwgs = p->nwg[st];  // workgroups of the launch
         int cs = 4;
-        while (cs < 20 && (nwg >> (cs + 1)) >= 8 * 64) cs++;
+        while (cs < 20 && (nwgs >> (cs + 1)) >= 8 * 64) cs++;
         p->index[st].chunk_shift = cs;
-        const int64_t turns = (nwg + ((int64_t)8 << cs) - 1) / ((int64_t)8 << cs);
+        const int64_t turns = (nwgs + ((int64_t)8 << cs) - 1) / ((int64_t)8 << cs);
         p->index[st].per_xcd = (int32_t)(turns << cs);
     }
     size_t bytes = nseg * sizeof(Seg);
@@ -341,8 +350,12 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes,
 
     }
     try {
-        if (p->nseg <= TFTQ_N_INLINE) deal_to_xcds(p, wgs);
-        else build_table(p, wgs);
+        if (p->nseg <= TFTQ_N_INLINE) {
+            deal_to_xcds(p, wgs);
+        } else if (const int rc = build_table(p, wgs)) {
+            delete p;
+            return rc;
+        }
     } catch (...) {
         delete p;
         return TFTQ_E_NOMEM;

@@ -728,6 +728,8 @@ DEV void reduce_rows_at_once(const Seg &s, const KParams &p, int j0, int lane, f
 template <bool GDIV, bool IEEE = false>
 DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 {
+    // a wavefront none of whose lanes has a row (rows go up with k) leaves at once
+    if (__builtin_amdgcn_ballot_w64(j0 + tid < s.slice_rows) == 0) return;
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     int64_t off[4];
 #pragma unroll
@@ -766,8 +768,14 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
     Seg s;
     int vb;
     if (!locate<INLINE, ST_R>(p, inl, s, vb)) return;
-    const int blk = vb - s.wg_begin[ST_R];
-    const int tid = threadIdx.x;
+    int blk = vb - s.wg_begin[ST_R];
+    int tid = threadIdx.x;
+    if (!INLINE && p.pieces) {
+        // vb is a quarter of a workgroup (tftq_reduce_pieces in tftq_internal.h): this wavefront is
+        // wavefront blk % 4 of workgroup blk / 4 of its tensor, whatever its neighbours work on
+        tid = (blk & 3) * 64 + (tid & 63);
+        blk >>= 2;
+    }
     const int ndw = (s.row_bytes >> 2) - 1;
     if (GDIV && p.div_mode == 3) {
         // averages over 1024 peers or more, not a power of two: the untuned path with plain divides
