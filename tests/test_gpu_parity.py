@@ -364,6 +364,30 @@ def test_average_over_a_very_large_group(q, oracle):
         full_check(q, oracle, peers, ws, ReduceOp.AVG, ranks=[0, ws // 2, ws - 1])
 
 
+@pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (2, ReduceOp.AVG), (3, ReduceOp.AVG), (4, ReduceOp.SUM),
+                                   (8, ReduceOp.AVG), (16, ReduceOp.SUM), (33, ReduceOp.AVG), (70, ReduceOp.AVG),
+                                   (1030, ReduceOp.AVG)])
+def test_group_sizes_on_long_lists(q, oracle, ws, op):
+    """Lists of more than 16 tensors: reduce numbers its work in quarters of workgroups, one
+    wavefront each, so wavefronts of one workgroup work on different tensors.  Every lane
+    mapping of reduce, tensors of one row and of many, empty tensors in between, rows that
+    take the plain divide, every group-size path (several rows at once for small groups,
+    coefficients through lanes, more peers than lanes, the plain-divide average)."""
+    g = torch.Generator().manual_seed(1000 + ws)
+    shapes = [(1, 40), (3, 12), (130,), (2, 100), (1, 200), (0, 7), (5, 400), (1, 700), (70, 3), (2, 2100),
+              (1, 4100), (9, 64), (300, 1), (1, 33), (2, 130), (700, 9), (1, 1030), (3, 260), (40, 40),
+              (1, 17000), (6, 520), (1, 5), (2, 2048)]
+    if ws > 100:
+        shapes = shapes[:19]
+    base = [[(torch.randn(s, generator=g) * (1 + p)).to(torch.bfloat16) for s in shapes] for p in range(min(ws, 5))]
+    for t in base[0]:
+        if t.dim() == 2 and t.shape[0] > 1:
+            t[1] *= 1e-30  # a scale beyond the fast division
+    peers = [base[p % len(base)] for p in range(ws)]
+    ranks = None if ws <= 4 else [0, ws // 2, ws - 1]
+    full_check(q, oracle, peers, ws, op, ranks)
+
+
 @pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (16, ReduceOp.AVG), (24, ReduceOp.SUM),
                                    (40, ReduceOp.AVG)])
 def test_short_rows_all_team_sizes(q, oracle, ws, op):
