@@ -34,6 +34,26 @@ DEV u32x4 load_codes(GLOBAL const u32 *payload, int d0, int ndw, int n)
     return w;
 }
 
+// The same without a branch, for the lanes that own a whole short row each (loads under a
+// condition end up one per basic block with a wait in front of each: a row of 3 dwords cost
+// its lane 3 round trips to memory per peer).  Four dword loads at indices clamped into the
+// row, then dwords past the end are cleared.
+DEV u32x4 load_codes_clamped(GLOBAL const u32 *payload, int d0, int ndw, int n)
+{
+    u32x4 w;
+    w.x = LOAD_STREAM(payload + min(d0, ndw - 1));
+    w.y = LOAD_STREAM(payload + min(d0 + 1, ndw - 1));
+    w.z = LOAD_STREAM(payload + min(d0 + 2, ndw - 1));
+    w.w = LOAD_STREAM(payload + min(d0 + 3, ndw - 1));
+    const int last = ndw - 1 - d0;  // position of the row's last dword in w
+    const u32 mask = (n & 3) ? (1u << (8 * (n & 3))) - 1u : 0xFFFFFFFFu;
+    w.x = last < 0 ? 0u : last == 0 ? w.x & mask : w.x;
+    w.y = last < 1 ? 0u : last == 1 ? w.y & mask : w.y;
+    w.z = last < 2 ? 0u : last == 2 ? w.z & mask : w.z;
+    w.w = last < 3 ? 0u : last == 3 ? w.w & mask : w.w;
+    return w;
+}
+
 DEV void store_codes(GLOBAL u32 *payload, int d0, int ndw, const u32x4 w)
 {
     const int rem = ndw - d0;
@@ -340,7 +360,13 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
         auto load_batch = [&](int k0) {
 #pragma unroll
             for (int b = 0; b < PB; b++) {
-                if (k0 + b < kend) {
+                if constexpr (TEAM == 1) {
+                    // no branch: a peer past the last one re-reads the last and is ignored below
+                    GLOBAL const u32 *prow = peer_row(p, min(k0 + b, kend - 1), off);
+                    sraw[b] = guarded_scale(prow);
+#pragma unroll
+                    for (int u = 0; u < UNITS; u++) w[b][u] = load_codes_clamped(prow + 1, u * 4, ndw, n);
+                } else if (k0 + b < kend) {
                     GLOBAL const u32 *prow = peer_row(p, k0 + b, off);
                     if (TEAM < 64) sraw[b] = guarded_scale(prow);
 #pragma unroll
