@@ -34,17 +34,18 @@ DEV u32x4 load_codes(GLOBAL const u32 *payload, int d0, int ndw, int n)
     return w;
 }
 
-// The same without a branch, for the lanes that own a whole short row each (loads under a
-// condition end up one per basic block with a wait in front of each: a row of 3 dwords cost
-// its lane 3 round trips to memory per peer).  Four dword loads at indices clamped into the
-// row, then dwords past the end are cleared.
+// The same without a branch, for lanes that own a whole short row each whose length is not a
+// whole number of 16-byte vectors (loads under a condition end up one per basic block with a
+// wait in front of each: a row of 3 dwords cost its lane 3 round trips to memory per peer):
+// four dword loads at indices clamped into the row, then dwords past the end are cleared.
+// Plain loads: the rows of neighbouring lanes share cache lines, as do the loads of one lane.
 DEV u32x4 load_codes_clamped(GLOBAL const u32 *payload, int d0, int ndw, int n)
 {
     u32x4 w;
-    w.x = LOAD_STREAM(payload + min(d0, ndw - 1));
-    w.y = LOAD_STREAM(payload + min(d0 + 1, ndw - 1));
-    w.z = LOAD_STREAM(payload + min(d0 + 2, ndw - 1));
-    w.w = LOAD_STREAM(payload + min(d0 + 3, ndw - 1));
+    w.x = payload[min(d0, ndw - 1)];
+    w.y = payload[min(d0 + 1, ndw - 1)];
+    w.z = payload[min(d0 + 2, ndw - 1)];
+    w.w = payload[min(d0 + 3, ndw - 1)];
     const int last = ndw - 1 - d0;  // position of the row's last dword in w
     const u32 mask = (n & 3) ? (1u << (8 * (n & 3))) - 1u : 0xFFFFFFFFu;
     w.x = last < 0 ? 0u : last == 0 ? w.x & mask : w.x;
@@ -331,7 +332,8 @@ DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float
 
 // Register-resident row: the team holds all accumulators of the row, each peer
 // row is read once.  UNITS = 16-byte vectors of codes per lane and peer.
-template <int TEAM, int UNITS, bool GDIV>
+// CLAMPED (one lane per row, rows that are not whole 16-byte vectors): loads without branches.
+template <int TEAM, int UNITS, bool GDIV, bool CLAMPED = false>
 DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 {
     constexpr int PB = 8 / UNITS;  // peers whose loads are in flight together
@@ -360,7 +362,7 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
         auto load_batch = [&](int k0) {
 #pragma unroll
             for (int b = 0; b < PB; b++) {
-                if constexpr (TEAM == 1) {
+                if constexpr (CLAMPED) {
                     // no branch: a peer past the last one re-reads the last and is ignored below
                     GLOBAL const u32 *prow = peer_row(p, min(k0 + b, kend - 1), off);
                     sraw[b] = guarded_scale(prow);
@@ -904,9 +906,15 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         break;
     }
     case K_GEN1:  // one lane per row: 1, 2 or 4 vectors of codes per peer
-        if (ndw <= 4) reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds);
-        else if (ndw <= 8) reduce_row<1, 2, GDIV>(s, p, blk * 256 + tid, 0, lds);
-        else reduce_row<1, 4, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        if (ndw & 3) {  // not whole 16-byte vectors
+            if (ndw <= 4) reduce_row<1, 1, GDIV, true>(s, p, blk * 256 + tid, 0, lds);
+            else if (ndw <= 8) reduce_row<1, 2, GDIV, true>(s, p, blk * 256 + tid, 0, lds);
+            else reduce_row<1, 4, GDIV, true>(s, p, blk * 256 + tid, 0, lds);
+        } else {
+            if (ndw <= 4) reduce_row<1, 1, GDIV>(s, p, blk * 256 + tid, 0, lds);
+            else if (ndw <= 8) reduce_row<1, 2, GDIV>(s, p, blk * 256 + tid, 0, lds);
+            else reduce_row<1, 4, GDIV>(s, p, blk * 256 + tid, 0, lds);
+        }
         break;
     case K_COL1: reduce_col1<GDIV>(s, p, blk * tftq_col1_rows_per_wg(ST_R), tid); break;
     default: break;
