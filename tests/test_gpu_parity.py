@@ -263,18 +263,21 @@ def test_dequantize_rows_through_lds_spans(q, oracle, dtype):
     """Contiguous rows that do not start and end on 64-byte boundaries are dequantized into
     LDS and written as one span per workgroup: row lengths on both sides of every team limit
     (512 B, 1, 2, 4, 8, 16 KB), row counts that leave the last workgroup partly filled,
-    destinations at every dword offset inside a 128-byte line (and at odd element offsets,
-    which take the direct path), guard elements around every destination, and scales outside
-    the range of the fast division in some rows."""
+    destinations at dword and at odd element offsets inside a 128-byte line, guard elements
+    around every destination, and scales outside the range of the fast division in some rows."""
     g = torch.Generator().manual_seed(23)
     esz = 4 if dtype == torch.float32 else 2
     cases = []  # (m, n, element offset of the destination)
-    for row_bytes in (68, 500, 516, 1000, 1028, 2000, 2052, 3000, 4092, 4100, 6000, 8188, 8196, 12000, 16380, 16388):
+    # (70 to 12002: 16-bit rows of an odd number of columns, whose spans start and end at even bytes only)
+    for row_bytes in (68, 70, 202, 500, 516, 1000, 1002, 1028, 2000, 2052, 3000, 3002, 4092, 4100, 6000, 6002, 8188,
+                      8196, 12000, 12002, 16380, 16388):
         n = row_bytes // esz
         for m, off in ((37, 0), (9, 2 * (4 // esz)), (70, 30 * (4 // esz) + 64), (3, 1)):
             cases.append((m, n, off))
     # rows of 1 to 31 whole vectors: several rows per lane, a workgroup's rows in two halves
-    for row_bytes, m in ((16, 5000), (48, 3), (48, 2500), (80, 1500), (144, 700), (272, 300), (400, 333), (496, 130)):
+    # (22 to 490: rows that are not whole vectors, 16-bit ones of an odd number of columns among them)
+    for row_bytes, m in ((16, 5000), (48, 3), (48, 2500), (80, 1500), (144, 700), (272, 300), (400, 333), (496, 130),
+                         (22, 3000), (36, 2000), (88, 1500), (120, 1100), (202, 800), (346, 400), (490, 150)):
         for off in (0, 4 // esz, 25 * (4 // esz), 1):
             cases.append((m, row_bytes // esz, off))
     cpu_src = []

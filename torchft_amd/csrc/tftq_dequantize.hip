@@ -128,8 +128,13 @@ DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS
                 for (int e = 0; e < 4; e++) o[4 + e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
             }
             if (idx < nvec) {
-                if constexpr (STAGED) *(LDS_AS u32x4_a4 *)(srow + 16 * idx) = Elem<T>::pack(o);
-                else STORE_STREAM(Elem<T>::pack(o), out + idx);
+                if constexpr (STAGED) {
+                    // (16-bit rows of an odd number of columns start at even bytes only)
+                    if (Elem<T>::ESZ == 4 || ((uint32_t)(uintptr_t)srow & 3u) == 0) *(LDS_AS u32x4_a4 *)(srow + 16 * idx) = Elem<T>::pack(o);
+                    else *(LDS_AS u32x4_a2 *)(srow + 16 * idx) = Elem<T>::pack(o);
+                } else {
+                    STORE_STREAM(Elem<T>::pack(o), out + idx);
+                }
             }
         }
         base += DV * TEAM;
@@ -140,7 +145,7 @@ DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS
 
 // The 256 / TEAM rows of a workgroup.  Rows that start and end on 64-byte boundaries are
 // written straight from the registers.  Other rows, when they are contiguous in memory
-// (row stride = row length) and dword-aligned, make one span of bytes per workgroup, which
+// (row stride = row length) and start at even bytes, make one span of bytes per workgroup, which
 // is assembled in LDS and written as whole lines (copy_out_span); that needs the span to fit
 // the stage, which the planner sees to for rows of up to 16 KB (pick_d_kind in tftq_plan.cpp).
 // What is left (longer rows, where the partial lines are few, and strided or oddly aligned
@@ -157,7 +162,7 @@ DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, u
     const bool few = s.n / Elem<T>::EPV <= 4 * TEAM;
     const int64_t rowb = (int64_t)s.n * Elem<T>::ESZ;
     // same branches for the whole workgroup
-    if (!rows_fill_lines<T>(s) && s.row_stride == s.n && ((s.ptr | (uint64_t)rowb) & 3u) == 0 &&
+    if (!rows_fill_lines<T>(s) && s.row_stride == s.n && ((s.ptr | (uint64_t)rowb) & 1u) == 0 &&
         R * rowb + 127 <= TFTQ_D_STAGE) {
         uint8_t *g0 = (uint8_t *)s.ptr + (int64_t)r0 * rowb;
         const int mis = (int)((uintptr_t)g0 & 127u);
@@ -237,16 +242,45 @@ DEV void dequantize_col1(const Seg &s, const KParams &p, int row0, int tid)
 }
 
 // K_VECS in dequantize: same shape as quantize_small, 8 vectors of codes and their
-// rows' scales in flight per lane.
+// rows' scales in flight per lane.  TAIL: the row is not a whole number of vectors; its last
+// vector is moved back to end with the row (it overlaps its neighbour, both store the same
+// values), so its codes start at any byte of the packed row.
+// First column of vector idx of a row of n columns.
+template <typename T>
+DEV int small_vec_col(int idx, int n)
+{
+    return min(idx * Elem<T>::EPV, n - Elem<T>::EPV);
+}
+
+// The EPV codes from column `col` on of the packed row `in`.  TAIL: they start at any byte
+// (gfx950 loads 4 and 8 bytes at any address).
+typedef u32 u32_a1 __attribute__((aligned(1)));
+typedef u32x2 u32x2_a1 __attribute__((aligned(1)));
+template <typename T, bool TAIL>
+DEV u32x2 load_small_codes(GLOBAL const u32 *in, int col)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    u32x2 w = {0u, 0u};
+    if constexpr (!TAIL) {
+        if constexpr (EPV == 4) w.x = LOAD_STREAM(in + 1 + (col >> 2));
+        else w = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + (col >> 2)));
+    } else {
+        GLOBAL const uint8_t *q = (GLOBAL const uint8_t *)in + 4 + col;
+        if constexpr (EPV == 4) w.x = LOAD_STREAM((GLOBAL const u32_a1 *)q);
+        else w = LOAD_STREAM((GLOBAL const u32x2_a1 *)q);
+    }
+    return w;
+}
+
 // Rows RBEG * teams .. REND * teams - 1 of the workgroup's rows.  STAGED: they are
 // neighbours in memory (row stride = row length) and go through the LDS stage as one span.
 template <typename T, int C, bool STAGED, bool POST, int RBEG, int REND>
 DEV void dequantize_small_rows(const Seg &s, const KParams &p, const SmallShape &h, const u32x2 (&w)[8 / C][C],
                                const float (&sc)[8 / C], bool fast, int row0, uint8_t *stage, int tid)
 {
-    constexpr int EPV = Elem<T>::EPV;
-    const int nvec = s.n / EPV;
-    const int rowb = nvec * 16;
+    constexpr int EPV = Elem<T>::EPV, ESZ = Elem<T>::ESZ;
+    const int nvec = tftq_small_nvec(s.n, ESZ);
+    const int rowb = s.n * ESZ;
     const int last = min(row0 + h.teams * (8 / C), s.m) - 1;
     const int first = row0 + RBEG * h.teams;
     if (first > last) return;  // same for the whole workgroup
@@ -256,7 +290,7 @@ DEV void dequantize_small_rows(const Seg &s, const KParams &p, const SmallShape 
     for (int r = RBEG; r < REND; r++) {
         const int row = row0 + r * h.teams + h.t;
         const DivCoef c = make_div(sc[r]);
-        GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)min(row, s.m - 1) * s.row_stride * Elem<T>::ESZ);
+        const uint64_t out = s.ptr + (uint64_t)((int64_t)min(row, s.m - 1) * s.row_stride * ESZ);
         LDS_AS uint8_t *srow = (LDS_AS uint8_t *)stage + mis + ((r - RBEG) * h.teams + h.t) * rowb;
 #pragma unroll
         for (int k = 0; k < C; k++) {
@@ -280,8 +314,13 @@ DEV void dequantize_small_rows(const Seg &s, const KParams &p, const SmallShape 
             }
             const int vec = k * h.team + h.l;
             if (row < s.m && vec < nvec) {
-                if constexpr (STAGED) *(LDS_AS u32x4_a4 *)(srow + 16 * vec) = Elem<T>::pack(o);
-                else STORE_STREAM(Elem<T>::pack(o), out + vec);
+                const int at = small_vec_col<T>(vec, s.n) * ESZ;  // bytes from the start of the row
+                if constexpr (STAGED) {
+                    if (((uint32_t)(uintptr_t)(srow + at) & 3u) == 0) *(LDS_AS u32x4_a4 *)(srow + at) = Elem<T>::pack(o);
+                    else *(LDS_AS u32x4_a2 *)(srow + at) = Elem<T>::pack(o);  // 16-bit rows of an odd number of columns
+                } else {
+                    STORE_STREAM(Elem<T>::pack(o), as_global<u32x4_a2>(out + (uint64_t)at));
+                }
             }
         }
     }
@@ -291,12 +330,11 @@ DEV void dequantize_small_rows(const Seg &s, const KParams &p, const SmallShape 
     }
 }
 
-template <typename T, int C, bool STAGED, bool POST>
+template <typename T, int C, bool STAGED, bool TAIL, bool POST>
 DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
-    constexpr int EPV = Elem<T>::EPV;
     constexpr int ROWS = 8 / C;  // 8, 4 or 2
-    const int nvec = s.n / EPV;
+    const int nvec = tftq_small_nvec(s.n, Elem<T>::ESZ);
     const int row0 = blk * (h.teams * ROWS);
     const float inv = 1.0f / (float)s.slice_rows;
 
@@ -308,15 +346,8 @@ DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, co
         GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr_fast(s, p.slot_size, min(row, s.m - 1), inv));
         sc[r] = as_f(in[0]);
 #pragma unroll
-        for (int k = 0; k < C; k++) {
-            const int idx = min(k * h.team + h.l, nvec - 1);
-            if constexpr (EPV == 4) {
-                w[r][k].x = LOAD_STREAM(in + 1 + idx);
-                w[r][k].y = 0;
-            } else {
-                w[r][k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
-            }
-        }
+        for (int k = 0; k < C; k++)  // a lane past the row's last vector re-reads that one and stores nothing
+            w[r][k] = load_small_codes<T, TAIL>(in, small_vec_col<T>(min(k * h.team + h.l, nvec - 1), s.n));
     }
     bool all_fast = true;
 #pragma unroll
@@ -328,21 +359,28 @@ DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, co
     dequantize_small_rows<T, C, STAGED, POST, ROWS / 2, ROWS>(s, p, h, w, sc, fast, row0, stage, tid);
 }
 
+template <typename T, bool STAGED, bool TAIL, bool POST>
+DEV void dequantize_small_s(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
+{
+    if (h.c == 1) dequantize_small_c<T, 1, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
+    else if (h.c == 2) dequantize_small_c<T, 2, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
+    else if (h.c == 3) dequantize_small_c<T, 3, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
+    else dequantize_small_c<T, 4, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
+}
+
 template <typename T, bool POST>
 DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
-    const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
-    // same branch for the whole workgroup
-    if (!rows_fill_lines<T>(s) && s.row_stride == s.n && (s.ptr & 3u) == 0) {
-        if (h.c == 1) dequantize_small_c<T, 1, true, POST>(s, p, blk, tid, h, stage);
-        else if (h.c == 2) dequantize_small_c<T, 2, true, POST>(s, p, blk, tid, h, stage);
-        else if (h.c == 3) dequantize_small_c<T, 3, true, POST>(s, p, blk, tid, h, stage);
-        else dequantize_small_c<T, 4, true, POST>(s, p, blk, tid, h, stage);
+    const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid);
+    const int rowb = s.n * Elem<T>::ESZ;
+    // same branches for the whole workgroup
+    const bool staged = !rows_fill_lines<T>(s) && s.row_stride == s.n && ((s.ptr | (uint64_t)rowb) & 1u) == 0;
+    if (s.n % Elem<T>::EPV) {
+        if (staged) dequantize_small_s<T, true, true, POST>(s, p, blk, tid, h, stage);
+        else dequantize_small_s<T, false, true, POST>(s, p, blk, tid, h, stage);
     } else {
-        if (h.c == 1) dequantize_small_c<T, 1, false, POST>(s, p, blk, tid, h, stage);
-        else if (h.c == 2) dequantize_small_c<T, 2, false, POST>(s, p, blk, tid, h, stage);
-        else if (h.c == 3) dequantize_small_c<T, 3, false, POST>(s, p, blk, tid, h, stage);
-        else dequantize_small_c<T, 4, false, POST>(s, p, blk, tid, h, stage);
+        if (staged) dequantize_small_s<T, true, false, POST>(s, p, blk, tid, h, stage);
+        else dequantize_small_s<T, false, false, POST>(s, p, blk, tid, h, stage);
     }
 }
 

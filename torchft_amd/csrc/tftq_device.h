@@ -461,7 +461,7 @@ DEV int64_t row_addr_fast(const Seg &s, int64_t slot_size, int row, float inv)
 // lines with every instruction.  The workgroup instead assembles the span in LDS, at the
 // offset that the span has inside its first 128-byte line, and then copies it out with
 // streaming 16-byte stores whose wavefronts each cover eight whole lines; only the first
-// and the last 16 bytes of the span can be partial and go out as dwords.
+// and the last 16 bytes of the span can be partial and go out as halfwords.
 #define LDS_AS __attribute__((address_space(3)))
 
 DEV void copy_out_span(const uint8_t *stage, uint8_t *g0, int len, int tid)
@@ -476,11 +476,12 @@ DEV void copy_out_span(const uint8_t *stage, uint8_t *g0, int len, int tid)
         const u32x4 v = *(const LDS_AS u32x4 *)(const LDS_AS uint8_t *)(stage + lo);
         if (lo >= mis && lo + 16 <= end) {
             STORE_STREAM(v, (GLOBAL u32x4 *)(line0 + lo));
-        } else {  // the span's first or last 16 bytes
+        } else {  // the span's first or last 16 bytes: halfwords (a span starts and ends at even bytes)
             const u32 w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int d = 0; d < 4; d++)
-                if (lo + 4 * d >= mis && lo + 4 * d < end) *(GLOBAL u32 *)(line0 + lo + 4 * d) = w[d];
+            for (int d = 0; d < 8; d++)
+                if (lo + 2 * d >= mis && lo + 2 * d < end)
+                    *(GLOBAL uint16_t *)(line0 + lo + 2 * d) = (uint16_t)(w[d >> 1] >> (16 * (d & 1)));
         }
     }
 }

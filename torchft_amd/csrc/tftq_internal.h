@@ -18,7 +18,7 @@ enum : int { ST_Q = 0, ST_R = 1, ST_D = 2 };
 // the packed buffer is contiguous and the GEN kinds only differ in team size.
 enum : uint8_t {
     K_NONE = 0,
-    K_VECS = 13,   // rows of 1-32 whole 16-byte vectors: 1 to 8 lanes per row, several rows per lane
+    K_VECS = 13,   // rows of 1-32 16-byte vectors (the last one moved back to end with the row): 1 to 8 lanes per row, several rows per lane
     K_VEC8 = 1,    // 8 lanes per row, 32 rows per workgroup
     K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
     K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
@@ -84,6 +84,13 @@ TFTQ_HD static inline void tftq_small_shape(int nvec, int *lt, int *c)
     *lt = t;
     *c = (nvec + (1 << t) - 1) >> t;
 }
+// vectors of a K_VECS row of n elements of esz bytes: whole ones, and one more that is moved
+// back to end with the row when n is not a multiple of the vector
+TFTQ_HD static inline int tftq_small_nvec(int n, int esz)
+{
+    const int epv = 16 / esz;
+    return (n + epv - 1) / epv;
+}
 static inline int tftq_small_rows_per_wg(int nvec)
 {
     int lt, c;
@@ -143,7 +150,7 @@ static_assert(sizeof(Seg) == 64, "Seg must be 64 bytes");
 static inline int tftq_rows_per_wg(const Seg &s, int st, int esz, int ws)
 {
     if (s.kind[st] == K_COL1) return tftq_col1_rows_per_wg(st);
-    if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(s.n / (16 / esz));
+    if (s.kind[st] == K_VECS) return tftq_small_rows_per_wg(tftq_small_nvec(s.n, esz));
     const int teams = TFTQ_WG / tftq_team_of(s.kind[st]);
     if (st == ST_R) return teams * tftq_reduce_rows_at_once(s.kind[st], s.row_bytes / 4 - 1, ws);
     return teams;

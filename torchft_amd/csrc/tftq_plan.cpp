@@ -68,8 +68,8 @@ static uint8_t pick_io_kind(const Seg &s, int esz)
     const bool vec_ok = s.col_stride == 1 && in_bytes >= 64;
     if (s.n == 1) return K_COL1;
     const int epv = 16 / esz;
-    if (s.col_stride == 1 && s.n % epv == 0 && s.n / epv >= 1 && s.n / epv <= 32)
-        return K_VECS;  // short rows of whole vectors
+    if (s.col_stride == 1 && s.n >= epv && tftq_small_nvec(s.n, esz) <= 32)
+        return K_VECS;  // short rows of at least one vector
     if (vec_ok) {
         // Team sizes measured on MI355X inside quantize -> reduce -> dequantize sequences (a
         // kernel's time depends on what ran before it, so loops over one kernel mislead):
@@ -95,7 +95,7 @@ static uint8_t pick_d_kind(const Seg &s, int esz)
     const uint8_t k = pick_io_kind(s, esz);
     const int64_t rowb = (int64_t)s.n * esz;
     if (k != K_VEC8 && k != K_VEC16 && k != K_VEC32 && k != K_VEC64 && k != K_VEC256) return k;
-    if (s.row_stride != s.n || (rowb & 3) != 0 || (rowb & 63) == 0 || rowb > 16384) return k;
+    if (s.row_stride != s.n || (rowb & 63) == 0 || rowb > 16384) return k;
     if (rowb <= 512) return K_VEC8;
     if (rowb <= 1024) return K_VEC16;
     if (rowb <= 2048) return K_VEC32;

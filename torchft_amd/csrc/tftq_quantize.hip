@@ -402,7 +402,42 @@ DEV void quantize_col1(const Seg &s, const KParams &p, int row0, int tid)
     }
 }
 
-// Short contiguous rows of whole 16-byte vectors (K_VECS, shape in tftq_device.h).
+// Short contiguous rows of 1 to 32 16-byte vectors (K_VECS, shape in tftq_device.h).  A row
+// whose length is not a whole number of vectors has its last vector moved back so that it
+// ends with the row: it overlaps its neighbour, whose elements count twice for the maximum
+// (no matter) and whose codes are written twice with the same values.
+// First column of vector idx of a row of n columns.
+template <typename T>
+DEV int small_vec_col(int idx, int n)
+{
+    return min(idx * Elem<T>::EPV, n - Elem<T>::EPV);
+}
+
+DEV void put8(LDS_AS uint8_t *q, u32 v) { *q = (uint8_t)v; }
+DEV void put8(GLOBAL uint8_t *q, u32 v) { *q = (uint8_t)v; }
+DEV void put32(LDS_AS uint8_t *q, u32 v) { *(LDS_AS u32 *)q = v; }
+DEV void put32(GLOBAL uint8_t *q, u32 v) { *(GLOBAL u32 *)q = v; }
+DEV void put64(LDS_AS uint8_t *q, u32x2 v) { *(LDS_AS u32x2_a4 *)q = v; }
+DEV void put64(GLOBAL uint8_t *q, u32x2 v) { *(GLOBAL u32x2_a4 *)q = v; }
+
+// The codes o of vector idx (of nv) into the packed row at `row` (LDS or global memory); the
+// lane of the last vector also clears the pad bytes behind the row's last code.
+template <typename T, typename P>
+DEV void put_small_codes(P row, int idx, int nv, int n, int row_bytes, const u32x2 o)
+{
+    constexpr int EPV = Elem<T>::EPV;
+    const int col = small_vec_col<T>(idx, n);
+    if ((col & 3) == 0) {
+        if constexpr (EPV == 4) put32(row + 4 + col, o.x);
+        else put64(row + 4 + col, o);
+    } else {  // the moved last vector of a row that is not a whole number of dwords
+#pragma unroll
+        for (int e = 0; e < EPV; e++) put8(row + 4 + col + e, (e < 4 ? o.x : o.y) >> (8 * (e & 3)));
+    }
+    if (idx == nv - 1)
+        for (int b = 4 + n; b < row_bytes; b++) put8(row + b, 0u);
+}
+
 // Scale of the row whose vectors a lane holds in v (maximum over the lanes of its team).
 template <typename T, int C>
 DEV float small_row_scale(const u32x4 (&v)[C], const SmallShape &h)
@@ -427,8 +462,7 @@ template <typename T, int C, int RBEG, int REND>
 DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)[8 / C][C], int row0, int last,
                              uint8_t *g0, uint8_t *stage, int tid)
 {
-    constexpr int EPV = Elem<T>::EPV;
-    const int nvec = s.n / EPV;
+    const int nvec = tftq_small_nvec(s.n, Elem<T>::ESZ);
     const int first = row0 + RBEG * h.teams;
     if (first > last) return;  // same for the whole workgroup
     uint8_t *gp = g0 + (int64_t)(RBEG * h.teams) * s.row_bytes;
@@ -439,21 +473,19 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
         const int row = row0 + r * h.teams + h.t;
         const float sc = small_row_scale<T, C>(v[r], h);
         if (row > last) continue;
-        LDS_AS u32 *srow = (LDS_AS u32 *)(LDS_AS uint8_t *)(stage + mis + ((r - RBEG) * h.teams + h.t) * s.row_bytes);
+        LDS_AS uint8_t *srow = (LDS_AS uint8_t *)(stage + mis + ((r - RBEG) * h.teams + h.t) * s.row_bytes);
         if (row >= s.m) {  // padding row: zero (:93-95 on a zero-filled buffer)
-            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) srow[d] = 0;
+            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) ((LDS_AS u32 *)srow)[d] = 0;
             continue;
         }
-        if (h.l == 0) srow[0] = as_u(sc);
+        if (h.l == 0) *(LDS_AS u32 *)srow = as_u(sc);
 #pragma unroll
         for (int k = 0; k < C; k++) {
             const int idx = k * h.team + h.l;
             if (idx >= nvec) continue;
             u32x4 x = v[r][k];
             if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // unpacked anew, not kept from the maximum
-            const u32x2 o = vec_codes<T>(x, sc);
-            if constexpr (EPV == 4) srow[1 + idx] = o.x;
-            else *(LDS_AS u32x2_a4 *)(srow + 1 + 2 * idx) = o;
+            put_small_codes<T>(srow, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
         }
     }
     __syncthreads();
@@ -466,9 +498,8 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
 template <typename T, int C>
 DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
-    constexpr int EPV = Elem<T>::EPV;
     constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane: 8, 4 or 2
-    const int nvec = s.n / EPV;
+    const int nvec = tftq_small_nvec(s.n, Elem<T>::ESZ);
     const int nrows = h.teams * ROWS;
     const int row0 = blk * nrows;
     const int m_pad = s.slice_rows * p.ws;
@@ -479,9 +510,12 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
     for (int r = 0; r < ROWS; r++) {
         const int row = row0 + r * h.teams + h.t;
         const int64_t e0 = (int64_t)min(row, s.m - 1) * s.row_stride;  // s.m >= 1: there are rows
-        GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + e0 * Elem<T>::ESZ);
 #pragma unroll
-        for (int k = 0; k < C; k++) v[r][k] = LOAD_STREAM(in + min(k * h.team + h.l, nvec - 1));
+        for (int k = 0; k < C; k++) {
+            // a lane past the row's last vector re-reads that one: a duplicate cannot change the maximum
+            const int col = small_vec_col<T>(min(k * h.team + h.l, nvec - 1), s.n);
+            v[r][k] = LOAD_STREAM(as_global<const u32x4_a2>(s.ptr + (e0 + col) * Elem<T>::ESZ));
+        }
     }
     {
         // the workgroup's rows that exist, row0 .. last, and the slot of the first one
@@ -507,18 +541,20 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
         const int row = row0 + r * h.teams + h.t;
         const float sc = small_row_scale<T, C>(v[r], h);
         if (row >= m_pad) continue;
-        GLOBAL u32 *out = as_global<u32>(p.packed + row_addr_fast(s, p.slot_size, row, inv));
+        GLOBAL uint8_t *out = as_global<uint8_t>(p.packed + row_addr_fast(s, p.slot_size, row, inv));
         if (row >= s.m) {
             // padding row: the reference leaves it zero (:93-95 on a zero-filled buffer)
-            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) out[d] = 0;
+            for (int d = h.l; d < (s.row_bytes >> 2); d += h.team) ((GLOBAL u32 *)out)[d] = 0;
             continue;
         }
-        if (h.l == 0) out[0] = as_u(sc);
+        if (h.l == 0) *(GLOBAL u32 *)out = as_u(sc);
 #pragma unroll
         for (int k = 0; k < C; k++) {
+            const int idx = k * h.team + h.l;
+            if (idx >= nvec) continue;
             u32x4 x = v[r][k];
             if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // as in quantize_small_span
-            if (k * h.team + h.l < nvec) vec_quant_store<T>(x, sc, out + 1, k * h.team + h.l);
+            put_small_codes<T>(out, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
         }
     }
 }
@@ -526,7 +562,7 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
 template <typename T>
 DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
-    const SmallShape h = small_shape(s.n / Elem<T>::EPV, tid);
+    const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid);
     if (h.c == 1) quantize_small_c<T, 1>(s, p, blk, tid, h, stage);
     else if (h.c == 2) quantize_small_c<T, 2>(s, p, blk, tid, h, stage);
     else if (h.c == 3) quantize_small_c<T, 3>(s, p, blk, tid, h, stage);
