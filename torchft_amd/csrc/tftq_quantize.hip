@@ -74,18 +74,14 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     u32x4 v[KMAX];
 #pragma unroll
     for (int k = 0; k < KMAX; k++) v[k] = LOAD_STREAM(in + min(k * TEAM + lane, nvec - 1));
-    float t[EPV - 1];
-    if (tail) {  // every lane reads the few tail elements; lane 0 will store their codes
-#pragma unroll
-        for (int e = 0; e < EPV - 1; e++) t[e] = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(e, tail - 1));
-    }
+    // the few elements after the last whole vector: lane e of the team takes element e (the
+    // lanes behind them re-read the last one), and later stores its code
+    float te = 0.0f;
+    if (tail) te = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(lane, tail - 1));
     float amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < KMAX; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
-    if (tail) {
-#pragma unroll
-        for (int e = 0; e < EPV - 1; e++) amax = fmaxf(amax, __builtin_fabsf(t[e]));
-    }
+    if (tail) amax = fmaxf(amax, __builtin_fabsf(te));
     amax = team_max<TEAM>(amax, lds);
     const float sc = calc_scale(amax);
     if (lane == 0) {
@@ -113,21 +109,12 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
             }
         }
     }
-    if (tail && lane == 0) {
-        float y[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) y[e] = (e < EPV - 1 && e < tail) ? t[e < EPV - 1 ? e : 0] * sc : 0.0f;
-        const int td = 1 + nvec * (EPV / 4);  // dword of the row that holds the first tail code
-        u32 w0 = pack_fp8x4(y[0], y[1], y[2], y[3]);
-        if (tail < 4) w0 &= (1u << (8 * tail)) - 1u;  // padding bytes are zero whatever 0 * sc gave
-        if (STAGED) srow[td] = w0;
-        else out[td] = w0;
-        if (EPV == 8 && tail > 4) {
-            u32 w1 = pack_fp8x4(y[4], y[5], y[6], y[7]);
-            if (tail < 8) w1 &= (1u << (8 * (tail - 4))) - 1u;
-            if (STAGED) srow[td + 1] = w1;
-            else out[td + 1] = w1;
-        }
+    // tail codes and the zero pad bytes behind them, one byte per lane (a team has at least 8 lanes)
+    if (tail && lane < s.row_bytes - 4 - nvec * EPV) {
+        const u32 b = lane < tail ? pack_fp8x4(te * sc, 0.0f, 0.0f, 0.0f) & 0xFFu : 0u;
+        const int at = 4 + nvec * EPV + lane;
+        if (STAGED) ((LDS_AS uint8_t *)srow)[at] = (uint8_t)b;
+        else ((GLOBAL uint8_t *)out)[at] = (uint8_t)b;
     }
 }
 
@@ -160,11 +147,8 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
     for (int k = 0; k < KR; k++) v[k] = LOAD_STREAM(in + min(k * TFTQ_WG + tid, nvec - 1));
 #pragma unroll
     for (int k = 0; k < G; k++) w[0][k] = LOAD_STREAM(in + min((KR + k) * TFTQ_WG + tid, nvec - 1));
-    float t[EPV - 1];
-    if (tail) {
-#pragma unroll
-        for (int e = 0; e < EPV - 1; e++) t[e] = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(e, tail - 1));
-    }
+    float te = 0.0f;  // lane e takes element e behind the last whole vector (see quantize_vec_k)
+    if (tail) te = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(tid, tail - 1));
     float amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < KR; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
@@ -181,10 +165,7 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
             park[(g * G + k) * TFTQ_WG + tid] = w[g & 1][k];
         }
     }
-    if (tail) {
-#pragma unroll
-        for (int e = 0; e < EPV - 1; e++) amax = fmaxf(amax, __builtin_fabsf(t[e]));
-    }
+    if (tail) amax = fmaxf(amax, __builtin_fabsf(te));
 #pragma nounroll
     for (int base = TFTQ_Q_VECS_LDS; base < nvec; base += 4 * TFTQ_WG) {  // first pass over the rest
         u32x4 x[4];
@@ -219,19 +200,9 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
             if (idx < nvec) vec_quant_store<T>(x[k], sc, out + 1, idx);
         }
     }
-    if (tail && tid == 0) {
-        float y[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) y[e] = (e < EPV - 1 && e < tail) ? t[e < EPV - 1 ? e : 0] * sc : 0.0f;
-        GLOBAL u32 *tw = out + 1 + nvec * (EPV / 4);
-        u32 w0 = pack_fp8x4(y[0], y[1], y[2], y[3]);
-        if (tail < 4) w0 &= (1u << (8 * tail)) - 1u;
-        tw[0] = w0;
-        if (EPV == 8 && tail > 4) {
-            u32 w1 = pack_fp8x4(y[4], y[5], y[6], y[7]);
-            if (tail < 8) w1 &= (1u << (8 * (tail - 4))) - 1u;
-            tw[1] = w1;
-        }
+    if (tail && tid < s.row_bytes - 4 - nvec * EPV) {  // tail codes and the zero pad bytes behind them
+        const u32 b = tid < tail ? pack_fp8x4(te * sc, 0.0f, 0.0f, 0.0f) & 0xFFu : 0u;
+        ((GLOBAL uint8_t *)out)[4 + nvec * EPV + tid] = (uint8_t)b;
     }
 }
 
