@@ -143,13 +143,81 @@ DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS
     }
 }
 
+// One workgroup per row, a row of more than 16 KB that does not start and end on 64-byte
+// boundaries: straight from the registers every wavefront's store would have partial blocks at
+// both ends ([6656, 32770] bf16: 155 us against 126 us for 32768 columns), so the row goes
+// through the LDS stage in pieces of 1024 vectors (16 KB), each written as whole lines; the
+// columns behind the last whole vector travel with the last piece.
+template <typename T, bool POST>
+DEV void dequantize_vec_pieces(const Seg &s, const KParams &p, int row, int tid, uint8_t *stage)
+{
+    constexpr int EPV = Elem<T>::EPV, ESZ = Elem<T>::ESZ, DV = 4, STEP = DV * TFTQ_WG;
+    if (row >= s.m) return;  // the whole workgroup
+    GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
+    const int nvec = s.n / EPV;
+    const DivCoef c = make_div(as_f(in[0]));
+    if (!c.fast) {  // same for all lanes
+        dequantize_gen<T, TFTQ_WG, POST>(s, p, row, tid);
+        return;
+    }
+    uint8_t *g_row = (uint8_t *)s.ptr + (int64_t)row * s.row_stride * ESZ;
+#pragma nounroll
+    for (int base = 0; base < nvec; base += STEP) {
+        u32x2 w[DV];
+#pragma unroll
+        for (int k = 0; k < DV; k++) {
+            const int idx = min(base + k * TFTQ_WG + tid, nvec - 1);
+            if constexpr (EPV == 4) {
+                w[k].x = LOAD_STREAM(in + 1 + idx);
+                w[k].y = 0;
+            } else {
+                w[k] = LOAD_STREAM((GLOBAL const u32x2_a4 *)(in + 1 + 2 * idx));
+            }
+        }
+        uint8_t *g0 = g_row + (int64_t)base * 16;
+        const int mis = (int)((uintptr_t)g0 & 127u);
+        LDS_AS uint8_t *sp = (LDS_AS uint8_t *)stage + mis;
+        const bool lastp = base + STEP >= nvec;
+        int len = min(STEP, nvec - base) * 16;
+        if (lastp) {  // the columns after the last whole vector, one element per lane
+            for (int col = nvec * EPV + tid; col < s.n; col += TFTQ_WG) {
+                const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
+                stage_elem<T>(sp, col - base * EPV, fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p));
+            }
+            len += (s.n - nvec * EPV) * ESZ;
+        }
+#pragma unroll
+        for (int k = 0; k < DV; k++) {
+            const int idx = base + k * TFTQ_WG + tid;
+            float o[EPV];
+            float f[4];
+            unpack_fp8x4(w[k].x, f);
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
+            if constexpr (EPV == 8) {
+                unpack_fp8x4(w[k].y, f);
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[4 + e] = fin<T, POST>(div_fast_signed(f[e], c.r, c.r_lo), p);
+            }
+            if (idx < nvec) {
+                LDS_AS uint8_t *at = sp + 16 * (idx - base);
+                if (ESZ == 4 || ((uint32_t)(uintptr_t)at & 3u) == 0) *(LDS_AS u32x4_a4 *)at = Elem<T>::pack(o);
+                else *(LDS_AS u32x4_a2 *)at = Elem<T>::pack(o);
+            }
+        }
+        __syncthreads();
+        copy_out_span(stage, g0, len, tid);
+        __syncthreads();  // before the next piece overwrites the stage
+    }
+}
+
 // The 256 / TEAM rows of a workgroup.  Rows that start and end on 64-byte boundaries are
 // written straight from the registers.  Other rows, when they are contiguous in memory
 // (row stride = row length) and start at even bytes, make one span of bytes per workgroup, which
 // is assembled in LDS and written as whole lines (copy_out_span); that needs the span to fit
 // the stage, which the planner sees to for rows of up to 16 KB (pick_d_kind in tftq_plan.cpp).
-// What is left (longer rows, where the partial lines are few, and strided or oddly aligned
-// rows) is written from the registers, partial blocks included.
+// Longer rows go through the stage a piece at a time (dequantize_vec_pieces).  What is left
+// (strided rows of up to 16 KB) is written from the registers, partial blocks included.
 template <typename T, int TEAM, bool POST>
 DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
@@ -173,6 +241,13 @@ DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, u
         __syncthreads();
         copy_out_span(stage, g0, len, tid);
         return;
+    }
+    if constexpr (TEAM == TFTQ_WG) {
+        if (!rows_fill_lines<T>(s) && ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ)) & 1u) == 0 &&
+            s.n / Elem<T>::EPV >= 1024) {
+            dequantize_vec_pieces<T, POST>(s, p, r0, tid, stage);
+            return;
+        }
     }
     if (few) dequantize_vec_k<T, TEAM, false, 4, POST>(s, p, r0 + team, lane, nullptr);
     else dequantize_vec_k<T, TEAM, false, 8, POST>(s, p, r0 + team, lane, nullptr);
