@@ -43,6 +43,20 @@ DEV void vec_quant_store(const u32x4 v, float s, GLOBAL u32 *payload, int idx)
     }
 }
 
+// Lanes past the last vector of a row re-read its last vector, moved down to a 16-byte
+// boundary when the row starts off one (the row has at least two vectors, so the bytes
+// are still the row's): whole wavefronts of such lanes then cost one aligned access, while
+// 64 copies of a vector at an odd 2-byte offset are served lane by lane (10001-column
+// bf16 rows, five vectors per lane needed and eight loaded: 153.8 us against 117.1 us for 10000).
+DEV int dup_vec_offset(GLOBAL const u32x4_a2 *in, int nvec)
+{
+    return (nvec - 1) * 16 - (int)((uintptr_t)in & 15u);
+}
+DEV GLOBAL const u32x4_a2 *vec_or_dup(GLOBAL const u32x4_a2 *in, int idx, int nvec, int dup)
+{
+    return (GLOBAL const u32x4_a2 *)((GLOBAL const uint8_t *)in + (idx < nvec ? idx * 16 : dup));
+}
+
 constexpr int Q_STAGE_BYTES = 16640;  // 8 rows of 2052 bytes (2048 16-bit columns) + 127 bytes of offset, rounded up (see copy_out_span)
 // the wide kernel, whose three workgroups per CU leave each 53 KB of LDS: one row of 32768 16-bit columns
 constexpr int Q_STAGE_BYTES_WIDE = 32912;
@@ -71,9 +85,10 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
     const int tail = s.n - nvec * EPV;  // elements after the last whole vector (rare)
     const int64_t r0 = (int64_t)row * s.row_stride;
     GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
+    const int dup = dup_vec_offset(in, nvec);
     u32x4 v[KMAX];
 #pragma unroll
-    for (int k = 0; k < KMAX; k++) v[k] = LOAD_STREAM(in + min(k * TEAM + lane, nvec - 1));
+    for (int k = 0; k < KMAX; k++) v[k] = LOAD_STREAM(vec_or_dup(in, k * TEAM + lane, nvec, dup));
     // the few elements after the last whole vector: lane e of the team takes element e (the
     // lanes behind them re-read the last one), and later stores its code
     float te = 0.0f;
@@ -142,11 +157,12 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
     const int tail = s.n - nvec * EPV;
     const int64_t r0 = (int64_t)row * s.row_stride;
     GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + r0 * Elem<T>::ESZ);
+    const int dup = dup_vec_offset(in, nvec);
     u32x4 v[KR], w[2][G];
 #pragma unroll
-    for (int k = 0; k < KR; k++) v[k] = LOAD_STREAM(in + min(k * TFTQ_WG + tid, nvec - 1));
+    for (int k = 0; k < KR; k++) v[k] = LOAD_STREAM(vec_or_dup(in, k * TFTQ_WG + tid, nvec, dup));
 #pragma unroll
-    for (int k = 0; k < G; k++) w[0][k] = LOAD_STREAM(in + min((KR + k) * TFTQ_WG + tid, nvec - 1));
+    for (int k = 0; k < G; k++) w[0][k] = LOAD_STREAM(vec_or_dup(in, (KR + k) * TFTQ_WG + tid, nvec, dup));
     float te = 0.0f;  // lane e takes element e behind the last whole vector (see quantize_vec_k)
     if (tail) te = Elem<T>::load(s.ptr, r0 + nvec * EPV + min(tid, tail - 1));
     float amax = 0.0f;
@@ -157,7 +173,7 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
         if (g + 1 < NG) {
 #pragma unroll
             for (int k = 0; k < G; k++)
-                w[(g + 1) & 1][k] = LOAD_STREAM(in + min((KR + (g + 1) * G + k) * TFTQ_WG + tid, nvec - 1));
+                w[(g + 1) & 1][k] = LOAD_STREAM(vec_or_dup(in, (KR + (g + 1) * G + k) * TFTQ_WG + tid, nvec, dup));
         }
 #pragma unroll
         for (int k = 0; k < G; k++) {
