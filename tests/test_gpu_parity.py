@@ -416,6 +416,35 @@ def test_short_rows_all_team_sizes(q, oracle, ws, op):
     full_check(q, oracle, half, ws, op, [ws // 2])
 
 
+@pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (8, ReduceOp.AVG), (16, ReduceOp.SUM),
+                                   (17, ReduceOp.AVG), (32, ReduceOp.SUM), (33, ReduceOp.AVG), (70, ReduceOp.SUM)])
+def test_rows_of_three_vectors_per_lane(q, oracle, ws, op):
+    """Rows of 513 ... 3072 columns: reduce gives rows that would leave more than a quarter of
+    a team idle to a team a quarter the size, three vectors of codes per lane (16 lanes for up
+    to 768 columns, 32 for up to 1536, 64 for up to 3072), when the group is no larger than
+    the team; group sizes on both sides of 16, 32 and 64, rows that end inside a vector or a
+    dword, row counts that leave teams of the last workgroup without a row, and rows whose
+    scale needs the plain divide."""
+    g = torch.Generator().manual_seed(300 + ws)
+    cols = [513, 516, 640, 700, 767, 768, 769, 1025, 1028, 1280, 1301, 1536, 1537, 2049, 2052, 2560, 2902, 3072, 3073]
+    rows = [ws + 3, 2 * ws + 1, 37]
+    shapes = [(rows[i % 3], c) for i, c in enumerate(cols)]
+    peers = []
+    for p in range(ws):
+        ts = []
+        for r, c in shapes:
+            x = torch.randn(r, c, generator=g) * (1 + p % 3)
+            x[1] *= 1e-30  # row scale beyond 2^64: the exact fallback
+            x[min(3, r - 1)] = 0.0
+            ts.append(x)
+        peers.append(ts)
+    ranks = None if ws <= 8 else [0, ws - 1]
+    full_check(q, oracle, peers, ws, op, ranks)
+    # one tensor per call: the plan with the segment table in the kernel arguments
+    for i in (2, 9, 15):
+        full_check(q, oracle, [[ts[i].to(torch.bfloat16)] for ts in peers], ws, op, [ws // 2])
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("ws", [1, 2, 8, 16])
 def test_short_rows_of_whole_vectors(q, oracle, dtype, ws):

@@ -104,7 +104,7 @@ static uint8_t pick_d_kind(const Seg &s, int esz)
     return K_VEC256;
 }
 
-static uint8_t pick_reduce_kind(const Seg &s)
+static uint8_t pick_reduce_kind(const Seg &s, int ws)
 {
     // one or two 16-byte vectors of codes per lane and peer, four for the longest rows
     const int ndw = s.row_bytes / 4 - 1;
@@ -112,8 +112,17 @@ static uint8_t pick_reduce_kind(const Seg &s)
     if (ndw <= 16) return K_GEN1;  // up to 64 bytes of codes: a lane per row beats a team with idle lanes
     if (ndw <= 32) return K_GEN8;
     if (ndw <= 64) return K_GEN16;
+    // Rows that would leave more than a quarter of the next team idle take three vectors per
+    // lane in a team a quarter the size (the fast path of a team holds a peer's division
+    // coefficients in a lane each: ws <= lanes).  2560 bf16 columns, 8 peers: 58.9 -> 48.1 us,
+    // 3072: 51.6 -> 47.9, 1280: 54.2 -> 49.9, 640: 59.1 -> 53.3.  (Not below 16 lanes: 8 lanes
+    // with three vectors each are slower than 32 with one, 384 columns: 62.5 against 55.5 us.)
     if (ndw <= 128) return K_GEN32;
+    if (ndw <= 192 && ws <= 16) return K_GEN16;
+    if (ndw <= 256) return K_GEN64;
+    if (ndw <= 384 && ws <= 32) return K_GEN32;
     if (ndw <= 512) return K_GEN64;
+    if (ndw <= 768 && ws <= 64) return K_GEN64;
     return K_GEN256;
 }
 
@@ -324,7 +333,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes,
 
         s.kind[ST_Q] = pick_io_kind(s, p->esz);
         s.kind[ST_D] = pick_d_kind(s, p->esz);
-        s.kind[ST_R] = pick_reduce_kind(s);
+        s.kind[ST_R] = pick_reduce_kind(s, p->ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
             const int64_t n = cdiv64(rows[st], tftq_rows_per_wg(s, st, p->esz, ws));

@@ -572,7 +572,7 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
 // the register cost of one peer.  The last peer is peeled off: nothing is loaded behind it.
 // Same requirements as reduce_rows.
 template <int TEAM, int UNITS, bool GDIV>
-DEV void reduce_rows_roll(const Seg &s, const KParams &p, int j, int lane, float *lds)
+DEV void reduce_rows_roll(const Seg &s, const KParams &p, int j, int lane, float *lds, bool valid = true)
 {
     const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
     const int ws = p.ws;
@@ -637,10 +637,10 @@ DEV void reduce_rows_roll(const Seg &s, const KParams &p, int j, int lane, float
 #pragma unroll
         for (int u = 0; u < UNITS; u++) {
             const u32x4 o = requant16<GDIV>(acc[u], s2, p);
-            if (4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)((GLOBAL uint8_t *)(orow + 1) + boff[u]) = o;
+            if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)((GLOBAL uint8_t *)(orow + 1) + boff[u]) = o;
         }
-        if (lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
-    } else {
+        if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+    } else if (valid) {
         reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
     }
 }
@@ -789,7 +789,7 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 }
 
 template <bool INLINE, bool GDIV, bool WIDE>
-__global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const InlineTable inl)
+__global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[16];
     __shared__ float parked[WIDE ? R_PARKED_CHUNKS * 16 * TFTQ_WG : 1];  // wide kernel: 48 KB (two workgroups per CU fit)
@@ -879,11 +879,14 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
             else reduce_rows_at_once<64, 2, 2, GDIV>(s, p, j, tid & 63, lds);
         } else if (p.ws > 64) {
             if (ndw <= 256) reduce_row<64, 1, GDIV>(s, p, j, tid & 63, lds);
-            else reduce_row<64, 2, GDIV>(s, p, j, tid & 63, lds);
+            else if (ndw <= 512) reduce_row<64, 2, GDIV>(s, p, j, tid & 63, lds);
+            else reduce_row_slow<64, GDIV>(s, p, j, tid & 63, lds);
         } else if (ndw <= 256) {
             reduce_rows<64, 1, true, GDIV>(s, p, j, tid & 63, lds);
-        } else {
+        } else if (ndw <= 512) {
             reduce_rows<64, 2, true, GDIV>(s, p, j, tid & 63, lds);
+        } else {
+            reduce_rows_roll<64, 3, GDIV>(s, p, j, tid & 63, lds);
         }
         break;
     }
@@ -894,7 +897,10 @@ __global__ __launch_bounds__(TFTQ_WG) void k_reduce(const KParams p, const Inlin
         auto small = [&](auto team_c) {
             constexpr int TEAM = decltype(team_c)::value;
             const int j = blk * (TFTQ_WG / TEAM) + tid / TEAM;
-            if (p.ws <= TEAM) {
+            if (ndw > 4 * TEAM) {  // three vectors per lane (see pick_reduce_kind)
+                if (p.ws <= TEAM) reduce_rows_roll<TEAM, 3, GDIV>(s, p, min(j, s.slice_rows - 1), tid % TEAM, lds, j < s.slice_rows);
+                else if (j < s.slice_rows) reduce_row_slow<TEAM, GDIV>(s, p, j, tid % TEAM, lds);
+            } else if (p.ws <= TEAM) {
                 reduce_rows<TEAM, 1, true, GDIV>(s, p, min(j, s.slice_rows - 1), tid % TEAM, lds, j < s.slice_rows);
             } else {
                 reduce_row<TEAM, 1, GDIV>(s, p, j, tid % TEAM, lds);
