@@ -792,6 +792,82 @@ def test_cfg4_full_size(q, oracle):
         same_bytes(outs[i], want[0], f"cfg4 dequantize tensor {i}")
 
 
+def test_buffers_beyond_four_gib(q, oracle):
+    """More than 2^32 elements in a tensor, rows and tensors at more than 2^32 bytes into a
+    slot and into the packed buffer (20.8 GB): a bf16 tensor [80000, 60000], a 1-D bf16 tensor
+    of 2 * 10^9 elements (8 packed bytes each) and a small tensor behind them, ws = 4.  All
+    three stages run at full size on the GPU; sampled rows (the first and last of slots, those
+    around element 2^31 and 2^32 and around byte 2^32 of a slot) are compared byte for byte
+    with the checker, which works on small buffers cut out of the full ones: a row's packed
+    bytes depend on that row alone, a reduced row on the ws rows at its place in the slots."""
+    ws, rank = 4, 3
+    dev_ = "cuda"
+    g = torch.Generator(device=dev_).manual_seed(5)
+    A = torch.empty(80000, 60000, dtype=torch.bfloat16, device=dev_)
+    for r0 in range(0, 80000, 8000):
+        A[r0:r0 + 8000].normal_(generator=g)
+        A[r0:r0 + 8000] *= 1 + r0 // 8000
+    B = torch.empty(2_000_000_000, dtype=torch.bfloat16, device=dev_)
+    for e0 in range(0, B.numel(), 250_000_000):
+        B[e0:e0 + 250_000_000].normal_(generator=g)
+        B[e0:e0 + 250_000_000] *= 1 + e0 // 250_000_000
+    C = torch.randn(5, 7, generator=g, device=dev_).to(torch.bfloat16)
+    tensors = [A, B, C]
+    shapes = [(80000, 60000), (B.numel(), 1), (5, 7)]
+    offs, slot, total = oracle.layout(shapes, ws)
+    assert offs[2] > 2 ** 32 and total == 4 * slot and total > 20 * 10 ** 9
+    srs = [-(-m // ws) for m, _ in shapes]
+    rbs = [(-(-n // 4) + 1) * 4 for _, n in shapes]
+    first_b = (2 ** 32 - offs[1]) // 8  # the row of B that starts at byte 2^32 of its slot
+    rows_a = sorted({0, 1, 19999, 20000, 20001, 2 ** 31 // 60000, 2 ** 31 // 60000 + 1, 59999, 60000,
+                     2 ** 32 // 60000, 2 ** 32 // 60000 + 1, 79998, 79999})
+    rows_b = sorted({0, 1, 255, 256, 2047, 2048, 499_999_999, 500_000_000, first_b - 1, first_b, first_b + 1,
+                     999_999_999, 1_000_000_000, 1_499_999_999, 1_500_000_000, 1_999_999_998, 1_999_999_999}
+                    | set(torch.randint(0, B.numel(), (500,), generator=torch.Generator().manual_seed(6)).tolist()))
+    picks = [rows_a, rows_b, list(range(5))]
+
+    def cut(buf, i, rows):
+        """The packed rows `rows` of tensor i out of a full packed buffer, as one uint8 tensor."""
+        at = torch.tensor([(r // srs[i]) * slot + offs[i] + (r % srs[i]) * rbs[i] for r in rows], device=dev_)
+        idx = at[:, None] + torch.arange(rbs[i], device=dev_)[None, :]
+        return buf[idx.view(-1)].cpu()
+
+    packed = q.fused_quantize_into_fp8(tensors, ws)
+    assert packed.numel() == total
+    small = [A[rows_a].cpu(), B[rows_b].cpu(), C.cpu()]
+    for i in range(3):
+        want = oracle.fused_quantize_into_fp8([small[i]], 1, nthreads=NT)
+        same_bytes(cut(packed, i, picks[i]), want[:len(picks[i]) * rbs[i]], f"quantize tensor {i}")
+
+    # Reduce on rank 3 of four different contributions: slot k of the receive buffer is slot
+    # (k + 1) % 4 of the packed buffer.  Row j of the slice is checked through a packed buffer
+    # of a tensor of ws * len(js) rows: its slot k holds the rows js of slot k.
+    recv = torch.cat([packed[((k + 1) % ws) * slot:((k + 1) % ws + 1) * slot] for k in range(ws)])
+    js = [sorted({r % srs[i] for r in picks[i]}) for i in range(3)]
+    js[2] = [0, 1]
+    minis = [torch.cat([cut(recv, i, [k * srs[i] + j for j in js[i]]) for k in range(ws)]) for i in range(3)]
+    q.fused_reduce_fp8(tensors, recv, ws, rank, ReduceOp.AVG)
+    for i in range(3):
+        like = torch.empty(ws * len(js[i]), shapes[i][1], dtype=torch.bfloat16)
+        oracle.fused_reduce_fp8([like], minis[i], ws, rank, ReduceOp.AVG, nthreads=NT)
+        nb = len(js[i]) * rbs[i]
+        same_bytes(cut(recv, i, [rank * srs[i] + j for j in js[i]]), minis[i][rank * nb:(rank + 1) * nb],
+                   f"reduce tensor {i}")
+
+    # Dequantize of that buffer (slot 3 reduced, the others as received)
+    outs = [torch.full_like(t, 7.0) for t in tensors]
+    q.fused_dequantize_from_fp8(outs, recv, ws)
+    for i in range(3):
+        rows = picks[i]
+        want = [torch.full((len(rows), shapes[i][1]), 7.0, dtype=torch.bfloat16)]
+        oracle.fused_dequantize_from_fp8(want, cut(recv, i, rows), 1, nthreads=NT)
+        got = outs[i][rows] if i != 1 else outs[i][rows].view(-1, 1)
+        same_bytes(got, want[0], f"dequantize tensor {i}")
+    # and nothing else: every element was written, the two big tensors are finite
+    assert not (outs[0] == 7.0).all(dim=1).any()
+    assert torch.isfinite(outs[1][::4099].float()).all()
+
+
 def test_cfg5_full_size(q, oracle):
     """All 10 000 ragged tensors, 16 peers, SUM: every peer's packed buffer, three
     ranks' reductions and the dequantized result against the checker."""
