@@ -840,7 +840,14 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
             if (ndw <= 1024) reduce_rows_at_once<256, 1, 2, GDIV>(s, p, j, tid, lds);
             else reduce_rows_at_once<256, 2, 2, GDIV>(s, p, j, tid, lds);
         } else if (WIDE && ndw > TFTQ_R_DWORDS && ndw <= TFTQ_R_DWORDS_WIDE && p.ws <= 64) {
-            reduce_rows<256, 8, false, GDIV>(s, p, j, tid, lds);
+            // vectors per lane and peer that this wavefront needs (see below): 4 to 8
+            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+            const int nu = min((ndw + 1023) >> 10, (ndw - 256 * wave + 1023) >> 10);
+            if (nu <= 4) reduce_rows_roll<256, 4, GDIV>(s, p, j, tid, lds);
+            else if (nu == 5) reduce_rows_roll<256, 5, GDIV>(s, p, j, tid, lds);
+            else if (nu == 6) reduce_rows_roll<256, 6, GDIV>(s, p, j, tid, lds);
+            else if (nu == 7) reduce_rows_roll<256, 7, GDIV>(s, p, j, tid, lds);
+            else reduce_rows_roll<256, 8, GDIV>(s, p, j, tid, lds);
         } else if (ndw > TFTQ_R_DWORDS) {
             if (p.ws > 64) reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
             else if (WIDE && ndw > TFTQ_R_DWORDS_WIDE) reduce_row_hybrid<GDIV>(s, p, j, tid, lds, parked);
