@@ -120,6 +120,22 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
             const int64_t rows = st == ST_Q ? m_pad : st == ST_R ? s.slice_rows : s.m;
             const int per_wg = tftq_rows_per_wg(s, st, dtype == TFTQ_F32 ? 4 : 2, ws);
             int64_t blocks = (rows + per_wg - 1) / per_wg;
+            if (st == ST_D) {  // long rows of dequantize are dealt to several workgroups
+                const int epv = dtype == TFTQ_F32 ? 4 : 8;
+                const int nvec = s.n / epv;
+                const int parts = s.kind[ST_D] == K_VEC256 && nvec > 2048 ? (nvec + 2043) / 2044 : 1;
+                bool ok = parts == tftq_d_row_parts(s.kind[ST_D], s.n, 16 / epv) && tftq_d_part_begin(nvec, parts, 0) == 0 &&
+                          tftq_d_part_begin(nvec, parts, parts) == nvec;
+                for (int k = 0; k < parts && ok && parts > 1; k++) {  // parts in order, none empty, none longer than a step
+                    const int a = tftq_d_part_begin(nvec, parts, k), b = tftq_d_part_begin(nvec, parts, k + 1);
+                    ok = a < b && b - a <= 2048 && (a & 3) == 0;
+                }
+                if (!ok) {
+                    printf("segment %d: %d parts for %d vectors\n", i, parts, nvec);
+                    return 1;
+                }
+                blocks *= parts;
+            }
             if (pieces) {
                 blocks = tftq_reduce_pieces(s, dtype == TFTQ_F32 ? 4 : 2, ws, blocks);
                 // every row of the tensor lies in one of its pieces
@@ -232,7 +248,7 @@ int main()
             const uint32_t kind = rnd() % 8;
             int64_t m, c;
             if (kind == 0) { m = rnd() % 5000; c = 1; }
-            else if (kind == 1) { m = rnd() % 40; c = 1 + rnd() % 20000; }
+            else if (kind == 1) { m = rnd() % 40; c = 1 + rnd() % 70000; }
             else if (kind == 2) { m = 0; c = rnd() % 9; }
             else { m = rnd() % 600; c = rnd() % 700; }
             s.push_back(m);

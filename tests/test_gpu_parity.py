@@ -526,6 +526,49 @@ def test_long_rows(q, oracle):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_rows_dealt_to_several_workgroups(q, oracle, dtype):
+    """Dequantize deals a row of more than 2048 vectors (8192 fp32 or 16384 16-bit columns) to
+    several workgroups: 2 to 130 parts, rows that fill
+    their 64-byte blocks and rows that do not (through LDS), rows at odd element offsets and
+    with gaps between them, columns behind the last whole vector, a row whose scale needs the
+    plain divide, guard elements around every destination."""
+    g = torch.Generator().manual_seed(77)
+    epv = 16 // torch.empty(0, dtype=dtype).element_size()
+    cols = [2049 * epv, 2048 * epv + 3, 4096 * epv, 4100 * epv - 1, 6007 * epv + epv // 2, 28672, 53250, 130 * 2044 * epv + 5]
+    tensors, guards = [], []
+    for i, c in enumerate(cols):
+        rows = 3 if c < 200000 else 2
+        if i % 3 == 1:  # a view with a gap of 5 elements between the rows, at an odd element offset
+            base = torch.full((rows * (c + 5) + 1,), 9.0, dtype=dtype)
+            t = base[1:].view(rows, c + 5)[:, :c]
+        else:
+            base = torch.full((rows * c + 2,), 9.0, dtype=dtype)
+            t = base[1:1 + rows * c].view(rows, c)
+        t.copy_((torch.randn(rows, c, generator=g) * (i + 1)).to(dtype))
+        if i == 2:
+            t[1] *= 1e-30
+        tensors.append(t)
+        guards.append(base)
+    ws = 2
+    packed_c = oracle.fused_quantize_into_fp8([t.clone() for t in tensors], ws, nthreads=NT)
+    bases_g = [b.cuda() for b in guards]
+    outs_g = []
+    for t, b, bg in zip(tensors, guards, bases_g):
+        off = t.storage_offset() - b.storage_offset()
+        outs_g.append(torch.as_strided(bg, t.shape, t.stride(), off))
+    same_bytes(q.fused_quantize_into_fp8(outs_g, ws), packed_c, "quantize")
+    for bg in bases_g:
+        bg.fill_(9.0)
+    q.fused_dequantize_from_fp8(outs_g, packed_c.cuda(), ws)
+    want = [torch.full_like(b, 9.0) for b in guards]
+    outs_c = [torch.as_strided(w, t.shape, t.stride(), t.storage_offset() - b.storage_offset())
+              for w, t, b in zip(want, tensors, guards)]
+    oracle.fused_dequantize_from_fp8(outs_c, packed_c, ws, nthreads=NT)
+    for i, (bg, w) in enumerate(zip(bases_g, want)):
+        same_bytes(bg, w, f"dequantize tensor {i} with its guard elements")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("ws", [1, 2, 3, 8])
 def test_single_column_tensors(q, oracle, dtype, ws):
     """1-D tensors (rows of one column): lengths around the rows a workgroup takes in each

@@ -70,19 +70,22 @@ DEV void dequantize_gen(const Seg &s, const KParams &p, int row, int lane)
 // and the first step's loads are on their way before the row's scale has arrived
 // and been turned into division coefficients.  STAGED: the row is written to its
 // place in LDS (srow) instead of global memory.
+// v0, v1: the row's vectors v0 ... v1 - 1 only (a row dealt to several workgroups,
+// tftq_d_row_parts); `last`: with the columns behind the last whole vector.
 template <typename T, int TEAM, bool STAGED, int DV, bool POST>
-DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS_AS uint8_t *srow)
+DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS_AS uint8_t *srow, int v0 = 0,
+                          int v1 = -1, bool last = true)
 {
     if (row >= s.m) return;
     GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
     constexpr int EPV = Elem<T>::EPV;
-    const int nvec = s.n / EPV;
+    const int nvec = v1 < 0 ? s.n / EPV : v1;
     const float sraw = as_f(in[0]);
     u32x2 w[DV];
     auto load_step = [&](int base) {
 #pragma unroll
         for (int k = 0; k < DV; k++) {
-            const int idx = min(base + k * TEAM + lane, nvec - 1);
+            const int idx = max(min(base + k * TEAM + lane, nvec - 1), 0);
             if constexpr (EPV == 4) {
                 w[k].x = LOAD_STREAM(in + 1 + idx);
                 w[k].y = 0;
@@ -91,7 +94,7 @@ DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS
             }
         }
     };
-    load_step(0);
+    load_step(v0);
     const DivCoef c = make_div(sraw);
     if (!c.fast) {  // same for all lanes of the team
         if constexpr (STAGED) {
@@ -100,20 +103,20 @@ DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS
                 const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
                 stage_elem<T>(srow, col, fin<T, POST>(f / c.s, p));
             }
-        } else {
+        } else if (v0 == 0) {  // the whole row, by the workgroup that has its first part
             dequantize_gen<T, TEAM, POST>(s, p, row, lane);
         }
         return;
     }
     GLOBAL u32x4_a2 *out = as_global<u32x4_a2>(s.ptr + (int64_t)row * s.row_stride * Elem<T>::ESZ);
     // the few columns after the last whole vector, one element per lane
-    for (int col = nvec * EPV + lane; col < s.n; col += TEAM) {
+    for (int col = (last ? nvec * EPV : s.n) + lane; col < s.n; col += TEAM) {
         const float f = __builtin_amdgcn_cvt_f32_fp8((int)((GLOBAL const uint8_t *)in)[4 + col], 0);
         const float v = fin<T, POST>(div_fast_signed(f, c.r, c.r_lo), p);
         if constexpr (STAGED) stage_elem<T>(srow, col, v);
         else Elem<T>::store(s.ptr, (int64_t)row * s.row_stride + col, v);
     }
-    for (int base = 0;;) {
+    for (int base = v0;;) {
 #pragma unroll
         for (int k = 0; k < DV; k++) {
             const int idx = base + k * TEAM + lane;
@@ -149,20 +152,20 @@ DEV void dequantize_vec_k(const Seg &s, const KParams &p, int row, int lane, LDS
 // through the LDS stage in pieces of 1024 vectors (16 KB), each written as whole lines; the
 // columns behind the last whole vector travel with the last piece.
 template <typename T, bool POST>
-DEV void dequantize_vec_pieces(const Seg &s, const KParams &p, int row, int tid, uint8_t *stage)
+DEV void dequantize_vec_pieces(const Seg &s, const KParams &p, int row, int tid, uint8_t *stage, int v0, int v1, bool last)
 {
     constexpr int EPV = Elem<T>::EPV, ESZ = Elem<T>::ESZ, DV = 4, STEP = DV * TFTQ_WG;
     if (row >= s.m) return;  // the whole workgroup
     GLOBAL const u32 *in = as_global<const u32>(p.packed + row_addr(s, p.slot_size, row));
-    const int nvec = s.n / EPV;
+    const int nvec = v1;  // this workgroup's vectors are v0 ... v1 - 1 of the row (see dequantize_vec_k)
     const DivCoef c = make_div(as_f(in[0]));
     if (!c.fast) {  // same for all lanes
-        dequantize_gen<T, TFTQ_WG, POST>(s, p, row, tid);
+        if (v0 == 0) dequantize_gen<T, TFTQ_WG, POST>(s, p, row, tid);
         return;
     }
     uint8_t *g_row = (uint8_t *)s.ptr + (int64_t)row * s.row_stride * ESZ;
 #pragma nounroll
-    for (int base = 0; base < nvec; base += STEP) {
+    for (int base = v0; base < nvec; base += STEP) {
         u32x2 w[DV];
 #pragma unroll
         for (int k = 0; k < DV; k++) {
@@ -177,7 +180,7 @@ DEV void dequantize_vec_pieces(const Seg &s, const KParams &p, int row, int tid,
         uint8_t *g0 = g_row + (int64_t)base * 16;
         const int mis = (int)((uintptr_t)g0 & 127u);
         LDS_AS uint8_t *sp = (LDS_AS uint8_t *)stage + mis;
-        const bool lastp = base + STEP >= nvec;
+        const bool lastp = last && base + STEP >= nvec;
         int len = min(STEP, nvec - base) * 16;
         if (lastp) {  // the columns after the last whole vector, one element per lane
             for (int col = nvec * EPV + tid; col < s.n; col += TFTQ_WG) {
@@ -225,10 +228,24 @@ DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, u
     const int r0 = blk * R;
     const int team = TEAM == 256 ? 0 : TEAM >= 64 ? __builtin_amdgcn_readfirstlane(tid / TEAM) : tid / TEAM;
     const int lane = tid & (TEAM - 1);
+    const int64_t rowb = (int64_t)s.n * Elem<T>::ESZ;
+    if constexpr (TEAM == TFTQ_WG) {
+        const int nvec = s.n / Elem<T>::EPV;
+        if (nvec > TFTQ_D_PART_VECS) {  // a part of a long row (tftq_d_row_parts)
+            const int parts = tftq_d_row_parts(K_VEC256, s.n, Elem<T>::ESZ);
+            const int row = blk / parts, part = blk - row * parts;
+            const int v0 = tftq_d_part_begin(nvec, parts, part), v1 = tftq_d_part_begin(nvec, parts, part + 1);
+            const bool last = part == parts - 1;
+            if (!rows_fill_lines<T>(s) && ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ)) & 1u) == 0)
+                dequantize_vec_pieces<T, POST>(s, p, row, tid, stage, v0, v1, last);
+            else if (v1 - v0 <= 4 * TEAM) dequantize_vec_k<T, TEAM, false, 4, POST>(s, p, row, lane, nullptr, v0, v1, last);
+            else dequantize_vec_k<T, TEAM, false, 8, POST>(s, p, row, lane, nullptr, v0, v1, last);
+            return;
+        }
+    }
     // DV = vectors a lane loads per step: 8 in flight where the row has them (4 is 1.3 % slower
     // on 4096-column bf16 rows), 4 for shorter rows, whose lanes would mostly load duplicates
     const bool few = s.n / Elem<T>::EPV <= 4 * TEAM;
-    const int64_t rowb = (int64_t)s.n * Elem<T>::ESZ;
     // same branches for the whole workgroup
     if (!rows_fill_lines<T>(s) && s.row_stride == s.n && ((s.ptr | (uint64_t)rowb) & 1u) == 0 &&
         R * rowb + 127 <= TFTQ_D_STAGE) {
@@ -245,7 +262,7 @@ DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, u
     if constexpr (TEAM == TFTQ_WG) {
         if (!rows_fill_lines<T>(s) && ((s.ptr | (uint64_t)(s.row_stride * Elem<T>::ESZ)) & 1u) == 0 &&
             s.n / Elem<T>::EPV >= 1024) {
-            dequantize_vec_pieces<T, POST>(s, p, r0, tid, stage);
+            dequantize_vec_pieces<T, POST>(s, p, r0, tid, stage, 0, s.n / Elem<T>::EPV, true);
             return;
         }
     }

@@ -156,6 +156,31 @@ static inline int tftq_rows_per_wg(const Seg &s, int st, int esz, int ws)
     return teams;
 }
 
+// Dequantize has no step that spans a row (the scale is there before the kernel starts), so
+// a row of the 256-lane kind with more vectors than one step of a workgroup takes (8 per
+// lane) is dealt to several workgroups, part after part: part k of a row of nvec vectors
+// starts at vector floor(k * nvec / parts), rounded down to a multiple of four (64 bytes),
+// none is empty or longer than one step, and the last one takes the columns behind the last
+// whole vector.  [7607, 28672] bf16: 127.9 us with one workgroup per row.
+constexpr int TFTQ_D_PART_VECS = 8 * TFTQ_WG;
+TFTQ_HD static inline int tftq_d_row_parts(uint8_t kind, int n, int esz)
+{
+    const int nvec = n / (16 / esz);
+    return kind == K_VEC256 && nvec > TFTQ_D_PART_VECS ? (nvec + TFTQ_D_PART_VECS - 5) / (TFTQ_D_PART_VECS - 4) : 1;
+}
+TFTQ_HD static inline int tftq_d_part_begin(int nvec, int parts, int part)
+{
+    return part >= parts ? nvec : (int)(((int64_t)part * nvec / parts) & ~(int64_t)3);
+}
+// Workgroups (or, in reduce on long lists, the workgroups that tftq_reduce_pieces turns into
+// pieces) of a segment with `rows` rows in a stage.
+static inline int64_t tftq_wgs_of(const Seg &s, int st, int esz, int ws, int64_t rows)
+{
+    const int per_wg = tftq_rows_per_wg(s, st, esz, ws);
+    const int64_t wgs = (rows + per_wg - 1) / per_wg;
+    return st == ST_D ? wgs * tftq_d_row_parts(s.kind[ST_D], s.n, esz) : wgs;
+}
+
 // Reduce on long lists (device table) numbers its work in quarters of workgroups, one
 // wavefront each, because most tensors of such lists have a row or two per slot and a
 // workgroup per tensor would be three quarters idle: wavefront w of workgroup v takes piece

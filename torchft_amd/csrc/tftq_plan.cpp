@@ -129,7 +129,8 @@ static uint8_t pick_reduce_kind(const Seg &s, int ws)
 // Bytes one workgroup of segment s moves in a stage.
 static double wg_weight(const Seg &s, int st, int esz, int ws)
 {
-    const double rows = (double)tftq_rows_per_wg(s, st, esz, ws);
+    double rows = (double)tftq_rows_per_wg(s, st, esz, ws);
+    if (st == ST_D) rows /= tftq_d_row_parts(s.kind[ST_D], s.n, esz);
     if (st == ST_R) return rows * (double)s.row_bytes * (ws + 1);
     return rows * ((double)s.n * esz + (double)s.row_bytes);
 }
@@ -336,7 +337,7 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes,
         s.kind[ST_R] = pick_reduce_kind(s, p->ws);
         const int64_t rows[3] = {m_pad, s.slice_rows, s.m};
         for (int st = 0; st < 3; st++) {
-            const int64_t n = cdiv64(rows[st], tftq_rows_per_wg(s, st, p->esz, ws));
+            const int64_t n = tftq_wgs_of(s, st, p->esz, ws, rows[st]);
             wgs[i][st] = (int32_t)n;
             wg[st] += n;
             if (wg[st] > INT32_MAX - 4096) {
