@@ -511,6 +511,13 @@ def test_rows_parked_in_lds(q, oracle):
         peers[1][0][1] *= 1e-30
         peers[0][1][2] = 0.0
         full_check(q, oracle, peers, 2, ReduceOp.AVG)
+    # Lists whose longest row parks one or two groups of five vectors per lane: the launch then has
+    # 32.9 or 40 KB of LDS instead of 60 (lengths at both ends of either range)
+    for dtype, cols in ((torch.bfloat16, [32776, 43008, 36864]), (torch.bfloat16, [43016, 53248, 33000]),
+                        (torch.float32, [16388, 21504]), (torch.float32, [21508, 26624, 100]),
+                        (torch.float16, [43015]), (torch.float16, [53255])):
+        peers = [[torch.randn(3, c, generator=g).to(dtype) * (p + 1) for c in cols] for p in range(2)]
+        full_check(q, oracle, peers, 2, ReduceOp.SUM)
 
 
 def test_long_rows(q, oracle):

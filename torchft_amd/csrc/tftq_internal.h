@@ -123,6 +123,13 @@ TFTQ_HD static inline int tftq_col1_rows_per_wg(int stage)
 // contain such rows.  What a row has beyond that is read twice.
 constexpr int TFTQ_Q_VECS = 8 * TFTQ_WG, TFTQ_Q_VECS_WIDE = 16 * TFTQ_WG;
 constexpr int TFTQ_Q_PARKED = 15;  // more vectors per lane that the wide quantize kernel parks in LDS (60 KB)
+constexpr int TFTQ_Q_PARK_GROUP = 5;  // they travel in groups of five; a row parks only the groups it needs
+// groups that a row of nvec vectors parks
+TFTQ_HD static inline int tftq_q_park_groups(int nvec)
+{
+    const int g = (nvec - TFTQ_Q_VECS_WIDE + TFTQ_Q_PARK_GROUP * TFTQ_WG - 1) / (TFTQ_Q_PARK_GROUP * TFTQ_WG);
+    return g < 0 ? 0 : g > TFTQ_Q_PARKED / TFTQ_Q_PARK_GROUP ? TFTQ_Q_PARKED / TFTQ_Q_PARK_GROUP : g;
+}
 constexpr int TFTQ_Q_VECS_LDS = TFTQ_Q_VECS_WIDE + TFTQ_Q_PARKED * TFTQ_WG;
 constexpr int TFTQ_R_DWORDS = 4096, TFTQ_R_DWORDS_WIDE = 8192;
 // Dequantize assembles rows that do not fill their 64-byte blocks in LDS, one span of bytes
@@ -246,7 +253,7 @@ struct tftq_plan {
     int64_t max_rows;
     int32_t nwg[3];
     bool wide[3];              // per stage: some row needs the kernel variant with more registers
-    bool parked;               // quantize: some row also needs the 60 KB of LDS (rows above TFTQ_Q_VECS_WIDE)
+    int parked;                // quantize: groups of 5 vectors per lane (20 KB of LDS each, up to 3) that the longest row parks in LDS (rows above TFTQ_Q_VECS_WIDE)
     Dealt dealt[3];            // inline table only
     int32_t dealt_per_xcd[3];  // inline table only: workgroups of the busiest XCD
     bool natural[3];           // inline table only: workgroup ids keep their order (see deal_to_xcds)

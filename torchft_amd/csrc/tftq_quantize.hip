@@ -143,7 +143,7 @@ DEV void quantize_vec_k(const Seg &s, const KParams &p, int row, int lane, float
 template <typename T>
 DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, float *lds, u32x4 *park)
 {
-    constexpr int KR = 2 * QV, G = 5, NG = TFTQ_Q_PARKED / G;
+    constexpr int KR = 2 * QV, G = TFTQ_Q_PARK_GROUP, NG = TFTQ_Q_PARKED / G;
     static_assert(NG * G == TFTQ_Q_PARKED, "groups of five");
     const bool active = row < s.slice_rows * p.ws;
     GLOBAL u32 *out = as_global<u32>(p.packed + (active ? row_addr(s, p.slot_size, row) : 0));
@@ -168,17 +168,21 @@ DEV void quantize_vec_lds(const Seg &s, const KParams &p, int row, int tid, floa
     float amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < KR; k++) amax = fmaxf(amax, vec_absmax<T>(v[k]));
+    // the groups this row needs (the launch has LDS for the longest row of the list)
+    const int ng = tftq_q_park_groups(nvec);
 #pragma unroll
     for (int g = 0; g < NG; g++) {
-        if (g + 1 < NG) {
+        if (g < ng) {  // same for the whole workgroup
+            if (g + 1 < NG && g + 1 < ng) {
 #pragma unroll
-            for (int k = 0; k < G; k++)
-                w[(g + 1) & 1][k] = LOAD_STREAM(vec_or_dup(in, (KR + (g + 1) * G + k) * TFTQ_WG + tid, nvec, dup));
-        }
+                for (int k = 0; k < G; k++)
+                    w[(g + 1) & 1][k] = LOAD_STREAM(vec_or_dup(in, (KR + (g + 1) * G + k) * TFTQ_WG + tid, nvec, dup));
+            }
 #pragma unroll
-        for (int k = 0; k < G; k++) {
-            amax = fmaxf(amax, vec_absmax<T>(w[g & 1][k]));
-            park[(g * G + k) * TFTQ_WG + tid] = w[g & 1][k];
+            for (int k = 0; k < G; k++) {
+                amax = fmaxf(amax, vec_absmax<T>(w[g & 1][k]));
+                park[(g * G + k) * TFTQ_WG + tid] = w[g & 1][k];
+            }
         }
     }
     if (tail) amax = fmaxf(amax, __builtin_fabsf(te));
@@ -564,9 +568,9 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 4 : 1) void k_quantize(const KParam
 {
     __shared__ float lds[4];
     __shared__ __align__(16) uint8_t stage_regular[WIDE ? 16 : Q_STAGE_BYTES];  // see copy_out_span
-    // Dynamic LDS of the wide kernel: Q_STAGE_BYTES_WIDE as its stage, or 60 KB when the plan has
-    // rows that are parked there (which limits a CU to two workgroups); a workgroup uses it
-    // for one or the other.
+    // Dynamic LDS of the wide kernel: Q_STAGE_BYTES_WIDE as its stage, or the 40 or 60 KB that the
+    // longest row of the plan parks there (which limits a CU to three or two workgroups); a
+    // workgroup uses it for one or the other.
     extern __shared__ u32x4 park[];
     uint8_t *stage = WIDE ? (uint8_t *)park : stage_regular;
     Seg s;
@@ -592,13 +596,13 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 4 : 1) void k_quantize(const KParam
 }
 
 template <typename T>
-static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, bool parked,
+static int launch_q(const KParams &kp, const InlineTable &inl, bool use_inline, bool wide, int parked,
                     hipStream_t st)
 {
     const unsigned grid = grid_of(kp);
     if (wide) {
-        const unsigned lds = parked ? TFTQ_Q_PARKED * TFTQ_WG * 16u : (unsigned)Q_STAGE_BYTES_WIDE;
-        static_assert(TFTQ_Q_PARKED * TFTQ_WG * 16 >= Q_STAGE_BYTES_WIDE, "the parking area also serves as the stage");
+        // the parking area also serves as the stage
+        const unsigned lds = std::max((unsigned)parked * TFTQ_Q_PARK_GROUP * TFTQ_WG * 16u, (unsigned)Q_STAGE_BYTES_WIDE);
         if (use_inline) return launch_kernel(k_quantize<T, true, true>, grid, lds, st, kp, inl);
         return launch_kernel(k_quantize<T, false, true>, grid, lds, st, kp, inl);
     }
