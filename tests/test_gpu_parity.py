@@ -417,32 +417,40 @@ def test_short_rows_all_team_sizes(q, oracle, ws, op):
 
 
 @pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (8, ReduceOp.AVG), (16, ReduceOp.SUM),
-                                   (17, ReduceOp.AVG), (32, ReduceOp.SUM), (33, ReduceOp.AVG), (70, ReduceOp.SUM)])
+                                   (17, ReduceOp.AVG), (32, ReduceOp.SUM), (33, ReduceOp.AVG), (64, ReduceOp.SUM),
+                                   (70, ReduceOp.AVG)])
 def test_rows_of_three_vectors_per_lane(q, oracle, ws, op):
-    """Rows of 513 ... 3072 columns: reduce gives rows that would leave more than a quarter of
-    a team idle to a team a quarter the size, three vectors of codes per lane (16 lanes for up
-    to 768 columns, 32 for up to 1536, 64 for up to 3072), when the group is no larger than
-    the team; group sizes on both sides of 16, 32 and 64, rows that end inside a vector or a
-    dword, row counts that leave teams of the last workgroup without a row, and rows whose
-    scale needs the plain divide."""
+    """Rows of 513 ... 3072 columns in tensors of at least 512 rows per rank: reduce gives rows
+    that would leave more than a quarter of a team idle to a team a quarter the size, three
+    vectors of codes per lane (16 lanes for up to 768 columns, 32 for up to 1536, 64 for up to
+    3072), when the group is no larger than the team; group sizes on both sides of 16, 32 and
+    64, rows that end inside a vector or a dword, row counts that leave teams of the last
+    workgroup without a row, rows whose scale needs the plain divide, and the same lengths
+    in tensors of a few rows, which keep the larger teams."""
     g = torch.Generator().manual_seed(300 + ws)
-    cols = [513, 516, 640, 700, 767, 768, 769, 1025, 1028, 1280, 1301, 1536, 1537, 2049, 2052, 2560, 2902, 3072, 3073]
-    rows = [ws + 3, 2 * ws + 1, 37]
-    shapes = [(rows[i % 3], c) for i, c in enumerate(cols)]
-    peers = []
-    for p in range(ws):
+    many = 512 * ws
+    shapes = [(5, c) for c in (513, 640, 767, 769, 1025, 1280, 1537, 2049, 2560, 3073)]
+    if ws <= 16:
+        shapes += [(many + 5, 516), (many + 1, 700), (many, 768)]
+    if ws <= 32:
+        shapes += [(many + 3, 1028), (many + 2, 1301), (many, 1536)]
+    if ws <= 64:
+        shapes += [(many + 7, 2052)] + ([(many + 1, 2902), (many, 3072)] if ws <= 17 else [])
+    base = []
+    for b in range(3):  # three different contributions, dealt to the peers in turn
         ts = []
         for r, c in shapes:
-            x = torch.randn(r, c, generator=g) * (1 + p % 3)
+            x = (torch.randn(r, c, generator=g) * (1 + b)).to(torch.bfloat16)
             x[1] *= 1e-30  # row scale beyond 2^64: the exact fallback
             x[min(3, r - 1)] = 0.0
             ts.append(x)
-        peers.append(ts)
-    ranks = None if ws <= 8 else [0, ws - 1]
+        base.append(ts)
+    peers = [base[p % 3] for p in range(ws)]
+    ranks = None if ws <= 2 else [0, ws - 1]
     full_check(q, oracle, peers, ws, op, ranks)
     # one tensor per call: the plan with the segment table in the kernel arguments
-    for i in (2, 9, 15):
-        full_check(q, oracle, [[ts[i].to(torch.bfloat16)] for ts in peers], ws, op, [ws // 2])
+    for i in (len(shapes) - 1, 10 if ws <= 64 else 3):
+        full_check(q, oracle, [[ts[i]] for ts in peers], ws, op, [ws // 2])
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
