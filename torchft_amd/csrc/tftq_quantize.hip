@@ -413,10 +413,16 @@ DEV void put64(GLOBAL uint8_t *q, u32x2 v) { *(GLOBAL u32x2_a4 *)q = v; }
 
 // The codes o of vector idx (of nv) into the packed row at `row` (LDS or global memory); the
 // lane of the last vector also clears the pad bytes behind the row's last code.
-template <typename T, typename P>
+// TAIL false: rows of whole vectors, which have neither a moved vector nor pad bytes.
+template <typename T, bool TAIL, typename P>
 DEV void put_small_codes(P row, int idx, int nv, int n, int row_bytes, const u32x2 o)
 {
     constexpr int EPV = Elem<T>::EPV;
+    if constexpr (!TAIL) {
+        if constexpr (EPV == 4) put32(row + 4 + idx * EPV, o.x);
+        else put64(row + 4 + idx * EPV, o);
+        return;
+    }
     const int col = small_vec_col<T>(idx, n);
     if ((col & 3) == 0) {
         if constexpr (EPV == 4) put32(row + 4 + col, o.x);
@@ -449,7 +455,7 @@ DEV float small_row_scale(const u32x4 (&v)[C], const SmallShape &h)
 
 // Rows RBEG * teams .. REND * teams - 1 of the workgroup's rows (those up to `last`)
 // through the LDS stage: g0 is the address of the workgroup's first packed row.
-template <typename T, int C, int RBEG, int REND>
+template <typename T, int C, bool TAIL, int RBEG, int REND>
 DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)[8 / C][C], int row0, int last,
                              uint8_t *g0, uint8_t *stage, int tid)
 {
@@ -476,7 +482,7 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
             if (idx >= nvec) continue;
             u32x4 x = v[r][k];
             if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // unpacked anew, not kept from the maximum
-            put_small_codes<T>(srow, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
+            put_small_codes<T, TAIL>(srow, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
         }
     }
     __syncthreads();
@@ -486,7 +492,7 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
 // The rows of a workgroup are neighbours; when they lie in one slot their packed rows are
 // one span of bytes, which goes through LDS (copy_out_span) in two halves (rows of 8 to 64
 // 16-bit columns make up to 24 KB per workgroup, more than the stage holds).
-template <typename T, int C>
+template <typename T, int C, bool TAIL>
 DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
     constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane: 8, 4 or 2
@@ -501,11 +507,17 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
     for (int r = 0; r < ROWS; r++) {
         const int row = row0 + r * h.teams + h.t;
         const int64_t e0 = (int64_t)min(row, s.m - 1) * s.row_stride;  // s.m >= 1: there are rows
+        // a lane past the row's last vector re-reads that one: a duplicate cannot change the maximum
+        if constexpr (TAIL) {
 #pragma unroll
-        for (int k = 0; k < C; k++) {
-            // a lane past the row's last vector re-reads that one: a duplicate cannot change the maximum
-            const int col = small_vec_col<T>(min(k * h.team + h.l, nvec - 1), s.n);
-            v[r][k] = LOAD_STREAM(as_global<const u32x4_a2>(s.ptr + (e0 + col) * Elem<T>::ESZ));
+            for (int k = 0; k < C; k++) {
+                const int col = small_vec_col<T>(min(k * h.team + h.l, nvec - 1), s.n);
+                v[r][k] = LOAD_STREAM(as_global<const u32x4_a2>(s.ptr + (e0 + col) * Elem<T>::ESZ));
+            }
+        } else {
+            GLOBAL const u32x4_a2 *in = as_global<const u32x4_a2>(s.ptr + e0 * Elem<T>::ESZ);
+#pragma unroll
+            for (int k = 0; k < C; k++) v[r][k] = LOAD_STREAM(in + min(k * h.team + h.l, nvec - 1));
         }
     }
     {
@@ -520,9 +532,9 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
             // common, the scales of all rows, in front of the branch (20 more registers)
             asm volatile("; rows through the stage");
             uint8_t *g0 = p.packed + (int64_t)slot0 * p.slot_size + s.slot_off + (int64_t)j0 * s.row_bytes;
-            quantize_small_span<T, C, 0, ROWS / 2>(s, h, v, row0, last, g0, stage, tid);
+            quantize_small_span<T, C, TAIL, 0, ROWS / 2>(s, h, v, row0, last, g0, stage, tid);
             __syncthreads();  // the first half has been copied out of the stage
-            quantize_small_span<T, C, ROWS / 2, ROWS>(s, h, v, row0, last, g0, stage, tid);
+            quantize_small_span<T, C, TAIL, ROWS / 2, ROWS>(s, h, v, row0, last, g0, stage, tid);
             return;
         }
     }
@@ -545,7 +557,7 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
             if (idx >= nvec) continue;
             u32x4 x = v[r][k];
             if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // as in quantize_small_span
-            put_small_codes<T>(out, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
+            put_small_codes<T, TAIL>(out, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
         }
     }
 }
@@ -554,10 +566,15 @@ template <typename T>
 DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
     const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid);
-    if (h.c == 1) quantize_small_c<T, 1>(s, p, blk, tid, h, stage);
-    else if (h.c == 2) quantize_small_c<T, 2>(s, p, blk, tid, h, stage);
-    else if (h.c == 3) quantize_small_c<T, 3>(s, p, blk, tid, h, stage);
-    else quantize_small_c<T, 4>(s, p, blk, tid, h, stage);
+    if (s.n % Elem<T>::EPV) {  // same for the whole workgroup
+        if (h.c == 1) quantize_small_c<T, 1, true>(s, p, blk, tid, h, stage);
+        else if (h.c == 2) quantize_small_c<T, 2, true>(s, p, blk, tid, h, stage);
+        else if (h.c == 3) quantize_small_c<T, 3, true>(s, p, blk, tid, h, stage);
+        else quantize_small_c<T, 4, true>(s, p, blk, tid, h, stage);
+    } else if (h.c == 1) quantize_small_c<T, 1, false>(s, p, blk, tid, h, stage);
+    else if (h.c == 2) quantize_small_c<T, 2, false>(s, p, blk, tid, h, stage);
+    else if (h.c == 3) quantize_small_c<T, 3, false>(s, p, blk, tid, h, stage);
+    else quantize_small_c<T, 4, false>(s, p, blk, tid, h, stage);
 }
 
 template <typename T, bool INLINE, bool WIDE>
