@@ -1077,12 +1077,20 @@ def test_random_tensor_lists(q, oracle, seed):
     op = rnd.choice([ReduceOp.SUM, ReduceOp.AVG])
     n_tensors = rnd.choice([1, 3, 9, 16, 17, 40])
     edges = [1, 2, 3, 4, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 260,
-             511, 512, 513, 520, 1023, 1024, 1025, 2047, 2048, 2049, 4095, 4096, 4100, 8191, 8192, 8200]
+             511, 512, 513, 520, 767, 768, 769, 1023, 1024, 1025, 1536, 1537, 2047, 2048, 2049, 3072, 3073,
+             4095, 4096, 4100, 8191, 8192, 8200]
+    # rows that dequantize deals to several workgroups, that quantize parks in LDS (one to three
+    # groups), that reduce takes in the wide variant
+    long_edges = [16383, 16384, 16392, 17001, 20000, 24580, 32768, 32776, 43008, 43016, 53250, 63500]
 
     def one_tensor():
         kind = rnd.random()
         n = rnd.choice(edges) if rnd.random() < 0.8 else rnd.randint(1, 9000)
         m = rnd.choice([0, 1, 2, 5, 16, 33, 70]) if n > 512 else rnd.choice([0, 1, 7, 64, 300, 1100])
+        if rnd.random() < 0.08:
+            n, m = rnd.choice(long_edges), rnd.choice([1, 2, 5])
+        elif 512 < n <= 3100 and ws <= 8 and rnd.random() < 0.15:
+            m = 512 * ws + rnd.randint(0, 9)  # rows enough for reduce's three-vectors-per-lane teams
         if kind < 0.1:
             return torch.randn(rnd.choice([1, 5, 1000, 4097]), generator=g)           # 1-D
         if kind < 0.2:
