@@ -463,7 +463,7 @@ DEV void dequantize_small_s(const Seg &s, const KParams &p, int blk, int tid, co
 template <typename T, bool POST>
 DEV void dequantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
-    const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid);
+    const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid, ST_D);
     const int rowb = s.n * Elem<T>::ESZ;
     // same branches for the whole workgroup
     const bool staged = !rows_fill_lines<T>(s) && s.row_stride == s.n && ((s.ptr | (uint64_t)rowb) & 1u) == 0;

@@ -423,17 +423,17 @@ DEV int64_t row_addr(const Seg &s, int64_t slot_size, int row)
 }
 
 // Short contiguous rows of whole 16-byte vectors (K_VECS; the shape is
-// tftq_small_shape): 1 to 8 lanes per row, and every lane works on several rows
+// tftq_small_shape): 1 to 8 lanes per row (up to 32 in dequantize), and every lane works on several rows
 // so that it has 8 loads in flight.  Row slot r of team t is row
 // row0 + r * teams + t: for a given r the teams of a wavefront read
 // consecutive rows, i.e. consecutive memory.
 struct SmallShape {
     int lt, c, team, teams, t, l;
 };
-DEV SmallShape small_shape(int nvec, int tid)
+DEV SmallShape small_shape(int nvec, int tid, int stage)
 {
     SmallShape h;
-    tftq_small_shape(nvec, &h.lt, &h.c);
+    tftq_small_shape(nvec, &h.lt, &h.c, stage);
     h.team = 1 << h.lt;
     h.teams = TFTQ_WG >> h.lt;
     h.t = tid >> h.lt;

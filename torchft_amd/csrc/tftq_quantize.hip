@@ -565,7 +565,7 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
 template <typename T>
 DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
-    const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid);
+    const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid, ST_Q);
     if (s.n % Elem<T>::EPV) {  // same for the whole workgroup
         if (h.c == 1) quantize_small_c<T, 1, true>(s, p, blk, tid, h, stage);
         else if (h.c == 2) quantize_small_c<T, 2, true>(s, p, blk, tid, h, stage);
