@@ -425,7 +425,7 @@ DEV void dequantize_small_rows(const Seg &s, const KParams &p, const SmallShape 
 template <typename T, int C, bool STAGED, bool TAIL, bool POST>
 DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
-    constexpr int ROWS = 8 / C;  // 8, 4 or 2
+    constexpr int ROWS = 8 / C;  // 8 or 4
     const int nvec = tftq_small_nvec(s.n, Elem<T>::ESZ);
     const int row0 = blk * (h.teams * ROWS);
     const float inv = 1.0f / (float)s.slice_rows;
@@ -454,10 +454,9 @@ DEV void dequantize_small_c(const Seg &s, const KParams &p, int blk, int tid, co
 template <typename T, bool STAGED, bool TAIL, bool POST>
 DEV void dequantize_small_s(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
+    // one or two vectors per lane (tftq_small_shape)
     if (h.c == 1) dequantize_small_c<T, 1, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
-    else if (h.c == 2) dequantize_small_c<T, 2, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
-    else if (h.c == 3) dequantize_small_c<T, 3, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
-    else dequantize_small_c<T, 4, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
+    else dequantize_small_c<T, 2, STAGED, TAIL, POST>(s, p, blk, tid, h, stage);
 }
 
 template <typename T, bool POST>

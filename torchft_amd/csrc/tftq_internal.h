@@ -70,21 +70,20 @@ TFTQ_HD static inline int tftq_reduce_rows_at_once(uint8_t kind, int ndw, int ws
     return 1;
 }
 
-// K_VECS: a row of nvec (1..32) 16-byte vectors is owned by a team of 2^lt lanes
-// (the smallest of 1, 2, 4, 8 that holds it with one vector per lane, else 8),
-// every lane holds c (1 to 4) vectors of it and works on 8 / c rows at once, so
-// that it has 6 to 8 loads in flight whatever the row length.  (Smaller teams
-// with more vectors per lane would leave fewer idle slots for some lengths,
-// 9 vectors as 4 x 3 for example, but measured slower: their loads cover
-// shorter runs of memory.)
-// Dequantize, which has no step that spans a row's lanes, takes teams of up to 16 lanes (rows
-// of up to 24 vectors) or 32 lanes (25 to 32 vectors): a team's loads and stores then cover
-// longer runs of memory.  256 bf16 columns: 133.6 us with 8 lanes of 4 vectors, 125.7 us with
-// 16 of 2, 120.4 us with 32 of 1; 200 columns: 154.8 / 135.8 / 129.6 us; 136 columns (17
-// vectors): 146.3 / 136.5 / 139.0 us; 100 fp32 columns: 239.3 / 215.5 / 220.1 us.
+// K_VECS: a row of nvec (1..32) 16-byte vectors is owned by a team of 2^lt lanes (the
+// smallest of 1, 2, 4, 8, 16 that holds it with one vector per lane; 16 lanes with two
+// vectors each for 17 to 24 vectors, 32 lanes for 25 to 32), every lane holds c (1 or 2)
+// vectors of it and works on 8 / c rows at once, so that it has 8 loads in flight whatever
+// the row length.  A team's loads and stores should cover long runs of memory: with at most
+// 8 lanes per row and up to 4 vectors per lane, 256 bf16 columns dequantized in 133.6 us
+// (16 lanes of 2: 125.7 us, 32 of 1: 120.4 us), 200 columns in 154.8 us (129.6 us), 100 fp32
+// columns in 239.3 us (220.0 us); quantize: 200 bf16 columns 128.9 -> 117.0 us, 136 columns
+// 125.3 -> 117.3 us, 100 fp32 columns 204.9 -> 188.4 us.  (17 vectors with 32 lanes: 139.0
+// against 136.5 us with 16 lanes of two.)
 TFTQ_HD static inline void tftq_small_shape(int nvec, int *lt, int *c, int stage = ST_Q)
 {
-    const int max_lt = stage != ST_D ? 3 : nvec >= 25 ? 5 : 4;
+    (void)stage;  // quantize and dequantize take the same teams
+    const int max_lt = nvec >= 25 ? 5 : 4;
     int t = 0;
     while (t < max_lt && (1 << t) < nvec) t++;
     *lt = t;

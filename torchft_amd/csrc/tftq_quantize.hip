@@ -443,13 +443,15 @@ DEV float small_row_scale(const u32x4 (&v)[C], const SmallShape &h)
 #pragma unroll
     for (int k = 0; k < C; k++) {
         a = fmaxf(a, vec_absmax<T>(v[k]));
-        // one vector after the other: with the 32 elements of four 16-bit vectors unpacked at
-        // once the kernel needs 81 registers instead of 70
-        if (C > 2) __builtin_amdgcn_sched_barrier(0);
     }
     if (h.lt >= 1) a = fmaxf(a, dpp_mov<0xB1>(a));   // quad_perm [1,0,3,2]
     if (h.lt >= 2) a = fmaxf(a, dpp_mov<0x4E>(a));   // quad_perm [2,3,0,1]
     if (h.lt >= 3) a = fmaxf(a, dpp_mov<0x141>(a));  // row_half_mirror
+    if (h.lt >= 4) a = fmaxf(a, dpp_mov<0x140>(a));  // row_mirror: all 16 lanes of a row agree
+    if (h.lt >= 5) {  // same for the whole workgroup
+        const float lo = fmaxf(bcast_lane(a, 0), bcast_lane(a, 16)), hi = fmaxf(bcast_lane(a, 32), bcast_lane(a, 48));
+        a = (threadIdx.x & 32) ? hi : lo;
+    }
     return calc_scale(a);
 }
 
@@ -480,8 +482,7 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
         for (int k = 0; k < C; k++) {
             const int idx = k * h.team + h.l;
             if (idx >= nvec) continue;
-            u32x4 x = v[r][k];
-            if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // unpacked anew, not kept from the maximum
+            const u32x4 x = v[r][k];
             put_small_codes<T, TAIL>(srow, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
         }
     }
@@ -495,7 +496,7 @@ DEV void quantize_small_span(const Seg &s, const SmallShape &h, const u32x4 (&v)
 template <typename T, int C, bool TAIL>
 DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, const SmallShape &h, uint8_t *stage)
 {
-    constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane: 8, 4 or 2
+    constexpr int ROWS = 8 / C;  // C vectors per lane and row, ROWS rows per lane: 8 or 4
     const int nvec = tftq_small_nvec(s.n, Elem<T>::ESZ);
     const int nrows = h.teams * ROWS;
     const int row0 = blk * nrows;
@@ -555,8 +556,7 @@ DEV void quantize_small_c(const Seg &s, const KParams &p, int blk, int tid, cons
         for (int k = 0; k < C; k++) {
             const int idx = k * h.team + h.l;
             if (idx >= nvec) continue;
-            u32x4 x = v[r][k];
-            if (C > 2) asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // as in quantize_small_span
+            const u32x4 x = v[r][k];
             put_small_codes<T, TAIL>(out, idx, nvec, s.n, s.row_bytes, vec_codes<T>(x, sc));
         }
     }
@@ -566,15 +566,12 @@ template <typename T>
 DEV void quantize_small(const Seg &s, const KParams &p, int blk, int tid, uint8_t *stage)
 {
     const SmallShape h = small_shape(tftq_small_nvec(s.n, Elem<T>::ESZ), tid, ST_Q);
-    if (s.n % Elem<T>::EPV) {  // same for the whole workgroup
+    // one or two vectors per lane (tftq_small_shape); same branch for the whole workgroup
+    if (s.n % Elem<T>::EPV) {
         if (h.c == 1) quantize_small_c<T, 1, true>(s, p, blk, tid, h, stage);
-        else if (h.c == 2) quantize_small_c<T, 2, true>(s, p, blk, tid, h, stage);
-        else if (h.c == 3) quantize_small_c<T, 3, true>(s, p, blk, tid, h, stage);
-        else quantize_small_c<T, 4, true>(s, p, blk, tid, h, stage);
+        else quantize_small_c<T, 2, true>(s, p, blk, tid, h, stage);
     } else if (h.c == 1) quantize_small_c<T, 1, false>(s, p, blk, tid, h, stage);
-    else if (h.c == 2) quantize_small_c<T, 2, false>(s, p, blk, tid, h, stage);
-    else if (h.c == 3) quantize_small_c<T, 3, false>(s, p, blk, tid, h, stage);
-    else quantize_small_c<T, 4, false>(s, p, blk, tid, h, stage);
+    else quantize_small_c<T, 2, false>(s, p, blk, tid, h, stage);
 }
 
 template <typename T, bool INLINE, bool WIDE>
