@@ -423,7 +423,7 @@ DEV int64_t row_addr(const Seg &s, int64_t slot_size, int row)
 }
 
 // Short contiguous rows of whole 16-byte vectors (K_VECS; the shape is
-// tftq_small_shape): 1 to 8 lanes per row (up to 32 in dequantize), and every lane works on several rows
+// tftq_small_shape): 1 to 32 lanes per row, and every lane works on several rows
 // so that it has 8 loads in flight.  Row slot r of team t is row
 // row0 + r * teams + t: for a given r the teams of a wavefront read
 // consecutive rows, i.e. consecutive memory.

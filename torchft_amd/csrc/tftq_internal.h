@@ -18,7 +18,7 @@ enum : int { ST_Q = 0, ST_R = 1, ST_D = 2 };
 // the packed buffer is contiguous and the GEN kinds only differ in team size.
 enum : uint8_t {
     K_NONE = 0,
-    K_VECS = 13,   // rows of 1-32 16-byte vectors (the last one moved back to end with the row): 1 to 8 lanes per row, several rows per lane
+    K_VECS = 13,   // rows of 1-32 16-byte vectors (the last one moved back to end with the row): 1 to 32 lanes per row, several rows per lane
     K_VEC8 = 1,    // 8 lanes per row, 32 rows per workgroup
     K_VEC16 = 11,  // 16 lanes per row, 16 rows per workgroup
     K_VEC32 = 12,  // 32 lanes per row, 8 rows per workgroup
