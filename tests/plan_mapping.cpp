@@ -123,12 +123,12 @@ static int check_plan(const std::vector<int64_t> &shapes, int ws, int dtype)
             if (st == ST_D) {  // long rows of dequantize are dealt to several workgroups
                 const int epv = dtype == TFTQ_F32 ? 4 : 8;
                 const int nvec = s.n / epv;
-                const int parts = s.kind[ST_D] == K_VEC256 && nvec > 2048 ? (nvec + 2043) / 2044 : 1;
+                const int parts = s.kind[ST_D] == K_VEC256 && nvec >= 1536 ? (nvec + 1023) / 1024 : 1;
                 bool ok = parts == tftq_d_row_parts(s.kind[ST_D], s.n, 16 / epv) && tftq_d_part_begin(nvec, parts, 0) == 0 &&
                           tftq_d_part_begin(nvec, parts, parts) == nvec;
                 for (int k = 0; k < parts && ok && parts > 1; k++) {  // parts in order, none empty, none longer than a step
                     const int a = tftq_d_part_begin(nvec, parts, k), b = tftq_d_part_begin(nvec, parts, k + 1);
-                    ok = a < b && b - a <= 2048 && (a & 3) == 0;
+                    ok = a < b && b - a <= 1024 + 3 && (a & 3) == 0;
                 }
                 if (!ok) {
                     printf("segment %d: %d parts for %d vectors\n", i, parts, nvec);

@@ -231,7 +231,7 @@ DEV void dequantize_vec_rows(const Seg &s, const KParams &p, int blk, int tid, u
     const int64_t rowb = (int64_t)s.n * Elem<T>::ESZ;
     if constexpr (TEAM == TFTQ_WG) {
         const int nvec = s.n / Elem<T>::EPV;
-        if (nvec > TFTQ_D_PART_VECS) {  // a part of a long row (tftq_d_row_parts)
+        if (nvec >= TFTQ_D_PART_MIN) {  // a part of a long row (tftq_d_row_parts)
             const int parts = tftq_d_row_parts(K_VEC256, s.n, Elem<T>::ESZ);
             const int row = blk / parts, part = blk - row * parts;
             const int v0 = tftq_d_part_begin(nvec, parts, part), v1 = tftq_d_part_begin(nvec, parts, part + 1);

@@ -169,16 +169,16 @@ static inline int tftq_rows_per_wg(const Seg &s, int st, int esz, int ws)
 }
 
 // Dequantize has no step that spans a row (the scale is there before the kernel starts), so
-// a row of the 256-lane kind with more vectors than one step of a workgroup takes (8 per
-// lane) is dealt to several workgroups, part after part: part k of a row of nvec vectors
-// starts at vector floor(k * nvec / parts), rounded down to a multiple of four (64 bytes),
-// none is empty or longer than one step, and the last one takes the columns behind the last
-// whole vector.  [7607, 28672] bf16: 127.9 us with one workgroup per row.
-constexpr int TFTQ_D_PART_VECS = 8 * TFTQ_WG;
+// a row of the 256-lane kind of 1536 vectors or more is dealt to several workgroups, part
+// after part, four vectors per lane or fewer each: part k of a row of nvec vectors starts at
+// vector floor(k * nvec / parts), rounded down to a multiple of four (64 bytes), none is
+// empty, and the last one takes the columns behind the last whole vector.  [7607, 28672]
+// bf16: 127.9 us with one workgroup per row, 116.1 us in parts of up to 2048 vectors.
+constexpr int TFTQ_D_PART_VECS = 4 * TFTQ_WG, TFTQ_D_PART_MIN = 6 * TFTQ_WG;
 TFTQ_HD static inline int tftq_d_row_parts(uint8_t kind, int n, int esz)
 {
     const int nvec = n / (16 / esz);
-    return kind == K_VEC256 && nvec > TFTQ_D_PART_VECS ? (nvec + TFTQ_D_PART_VECS - 5) / (TFTQ_D_PART_VECS - 4) : 1;
+    return kind == K_VEC256 && nvec >= TFTQ_D_PART_MIN ? (nvec + TFTQ_D_PART_VECS - 1) / TFTQ_D_PART_VECS : 1;
 }
 TFTQ_HD static inline int tftq_d_part_begin(int nvec, int parts, int part)
 {

@@ -95,7 +95,19 @@ static uint8_t pick_d_kind(const Seg &s, int esz)
     const uint8_t k = pick_io_kind(s, esz);
     const int64_t rowb = (int64_t)s.n * esz;
     if (k != K_VEC8 && k != K_VEC16 && k != K_VEC32 && k != K_VEC64 && k != K_VEC256) return k;
-    if (s.row_stride != s.n || (rowb & 63) == 0 || rowb > 16384) return k;
+    if (s.row_stride != s.n || (rowb & 63) == 0 || rowb > 16384) {
+        // Written from the registers: about three to six vectors per lane (more lanes with fewer
+        // vectors each cover longer runs of memory per instruction; below three the lanes have
+        // too little in flight).  8 KB rows: 116.3 us with 64 lanes of 8 vectors, 110.8 us with
+        // 128 of 4; 4 KB: 117.3 -> 111.3 us; 3 KB: 118.5 -> 110.9 us; 5 KB as 128 x 2.5: 105.5
+        // against 102.3 us with 64 x 5; 2 KB as 64 x 2: 115.7 against 114.3 us with 32 x 4.
+        // (10 KB rows: 111.9 us with 256 lanes of 2.5 vectors, 115.7 us with 128 of 5.)
+        const int64_t nvec = rowb / 16;
+        if (nvec > 512) return K_VEC256;
+        if (nvec >= 384) return K_VEC128;
+        if (nvec >= 192) return K_VEC64;
+        return k;
+    }
     if (rowb <= 512) return K_VEC8;
     if (rowb <= 1024) return K_VEC16;
     if (rowb <= 2048) return K_VEC32;
