@@ -48,7 +48,9 @@ typedef u32x2 u32x2_a4 __attribute__((aligned(4)));
 #define GLOBAL __attribute__((address_space(1)))
 
 enum { C_RO = 0, C_WO = 1, C_R2W1 = 2, C_R1W2 = 3, C_R4W1 = 4, C_R1W4 = 5, C_R8W1 = 6,
-       C_RED = 7, C_RED_LINE = 8, C_DEQ = 9, C_QNT = 10, C_KINDS = 11 };
+       C_RED = 7, C_RED_LINE = 8, C_DEQ = 9, C_QNT = 10,
+       // the four mixes of quantize and dequantize with 4 steps per lane instead of 8
+       C_R2W1_4 = 11, C_R1W2_4 = 12, C_R4W1_4 = 13, C_R1W4_4 = 14, C_KINDS = 15 };
 
 template <typename V, bool NT>
 __device__ __forceinline__ V ld(GLOBAL const V *p)
@@ -62,61 +64,61 @@ __device__ __forceinline__ void st(V v, GLOBAL V *p)
     else *p = v;
 }
 
-// RV / WV: bytes a lane reads / writes per step (8 steps per chunk); WV == 2 stands for one
-// 16-byte store per 8 loads.
-template <int RV, int WV, bool NTL, bool NTS>
+// RV / WV: bytes a lane reads / writes per step (STEPS steps per chunk: all its loads, then
+// all its stores); WV == 2 stands for one 16-byte store per 8 loads.
+template <int RV, int WV, bool NTL, bool NTS, int STEPS = 8>
 __global__ __launch_bounds__(256) void k_stream(const uint8_t *src, uint8_t *dst, int64_t chunks, u32 never)
 {
     const int64_t c = blockIdx.x;
     if (c >= chunks) return;
     const int t = threadIdx.x;
-    u32 x[8][4];
+    u32 x[STEPS][4];
 #pragma unroll
-    for (int k = 0; k < 8; k++) x[k][0] = x[k][1] = x[k][2] = x[k][3] = (u32)t + k;
+    for (int k = 0; k < STEPS; k++) x[k][0] = x[k][1] = x[k][2] = x[k][3] = (u32)t + k;
     if constexpr (RV == 16) {
-        GLOBAL const u32x4 *s = (GLOBAL const u32x4 *)(uint64_t)(src + c * (8 * 256 * 16));
+        GLOBAL const u32x4 *s = (GLOBAL const u32x4 *)(uint64_t)(src + c * (STEPS * 256 * 16));
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
+        for (int k = 0; k < STEPS; k++) {
             const u32x4 v = ld<u32x4, NTL>(s + k * 256 + t);
             x[k][0] = v.x; x[k][1] = v.y; x[k][2] = v.z; x[k][3] = v.w;
         }
     } else if constexpr (RV == 8) {
-        GLOBAL const u32x2 *s = (GLOBAL const u32x2 *)(uint64_t)(src + c * (8 * 256 * 8));
+        GLOBAL const u32x2 *s = (GLOBAL const u32x2 *)(uint64_t)(src + c * (STEPS * 256 * 8));
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
+        for (int k = 0; k < STEPS; k++) {
             const u32x2 v = ld<u32x2, NTL>(s + k * 256 + t);
             x[k][0] = v.x; x[k][1] = v.y; x[k][2] = v.x ^ 1u; x[k][3] = v.y ^ 1u;
         }
     } else if constexpr (RV == 4) {
-        GLOBAL const u32 *s = (GLOBAL const u32 *)(uint64_t)(src + c * (8 * 256 * 4));
+        GLOBAL const u32 *s = (GLOBAL const u32 *)(uint64_t)(src + c * (STEPS * 256 * 4));
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
+        for (int k = 0; k < STEPS; k++) {
             const u32 v = ld<u32, NTL>(s + k * 256 + t);
             x[k][0] = v; x[k][1] = v ^ 1u; x[k][2] = v ^ 2u; x[k][3] = v ^ 3u;
         }
     }
     if constexpr (WV == 16) {
-        GLOBAL u32x4 *d = (GLOBAL u32x4 *)(uint64_t)(dst + c * (8 * 256 * 16));
+        GLOBAL u32x4 *d = (GLOBAL u32x4 *)(uint64_t)(dst + c * (STEPS * 256 * 16));
 #pragma unroll
-        for (int k = 0; k < 8; k++) st<u32x4, NTS>(u32x4{x[k][0], x[k][1], x[k][2], x[k][3]}, d + k * 256 + t);
+        for (int k = 0; k < STEPS; k++) st<u32x4, NTS>(u32x4{x[k][0], x[k][1], x[k][2], x[k][3]}, d + k * 256 + t);
     } else if constexpr (WV == 8) {
-        GLOBAL u32x2 *d = (GLOBAL u32x2 *)(uint64_t)(dst + c * (8 * 256 * 8));
+        GLOBAL u32x2 *d = (GLOBAL u32x2 *)(uint64_t)(dst + c * (STEPS * 256 * 8));
 #pragma unroll
-        for (int k = 0; k < 8; k++) st<u32x2, NTS>(u32x2{x[k][0] ^ x[k][1], x[k][2] ^ x[k][3]}, d + k * 256 + t);
+        for (int k = 0; k < STEPS; k++) st<u32x2, NTS>(u32x2{x[k][0] ^ x[k][1], x[k][2] ^ x[k][3]}, d + k * 256 + t);
     } else if constexpr (WV == 4) {
-        GLOBAL u32 *d = (GLOBAL u32 *)(uint64_t)(dst + c * (8 * 256 * 4));
+        GLOBAL u32 *d = (GLOBAL u32 *)(uint64_t)(dst + c * (STEPS * 256 * 4));
 #pragma unroll
-        for (int k = 0; k < 8; k++) st<u32, NTS>(x[k][0] ^ x[k][1] ^ x[k][2] ^ x[k][3], d + k * 256 + t);
+        for (int k = 0; k < STEPS; k++) st<u32, NTS>(x[k][0] ^ x[k][1] ^ x[k][2] ^ x[k][3], d + k * 256 + t);
     } else if constexpr (WV == 2) {
         u32x4 a = {0, 0, 0, 0};
 #pragma unroll
-        for (int k = 0; k < 8; k++) a ^= u32x4{x[k][0], x[k][1], x[k][2], x[k][3]};
+        for (int k = 0; k < STEPS; k++) a ^= u32x4{x[k][0], x[k][1], x[k][2], x[k][3]};
         GLOBAL u32x4 *d = (GLOBAL u32x4 *)(uint64_t)(dst + c * (256 * 16));
         st<u32x4, NTS>(a, d + t);
     } else {  // read only: the loads must not be optimised away
         u32 a = 0;
 #pragma unroll
-        for (int k = 0; k < 8; k++) a ^= x[k][0] ^ x[k][1] ^ x[k][2] ^ x[k][3];
+        for (int k = 0; k < STEPS; k++) a ^= x[k][0] ^ x[k][1] ^ x[k][2] ^ x[k][3];
         if (a == never) *(GLOBAL u32 *)(uint64_t)dst = a;
     }
 }
@@ -241,6 +243,9 @@ extern "C" int tftq_ceiling_bytes(int kind, int64_t units, int row_bytes, int64_
     } else if (kind == C_RED || kind == C_RED_LINE) {
         *read_bytes = units * (int64_t)row_bytes * 8;
         *write_bytes = units * (int64_t)row_bytes;
+    } else if (kind >= C_R2W1_4) {
+        *read_bytes = units * 4 * 256 * (int64_t)rv[kind - C_R2W1_4 + C_R2W1];
+        *write_bytes = units * 4 * 256 * (int64_t)wv[kind - C_R2W1_4 + C_R2W1];
     } else {
         *read_bytes = units * 8 * 256 * (int64_t)rv[kind];
         *write_bytes = units * 8 * 256 * (int64_t)wv[kind];
@@ -265,12 +270,13 @@ extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t
     if (units <= 0) return 0;
     if (units > 0x7FFFFFF0) return -1;
     const dim3 grid((unsigned)units);
-#define TFTQ_C(RV, WV)                                                                                     \
+#define TFTQ_C(RV, WV) TFTQ_CS(RV, WV, 8)
+#define TFTQ_CS(RV, WV, STEPS)                                                                             \
     do {                                                                                                   \
-        if (nt_loads && nt_stores) hipLaunchKernelGGL((k_stream<RV, WV, true, true>), grid, block, 0, s, a, b, units, 0x9E3779B9u);  \
-        else if (nt_loads) hipLaunchKernelGGL((k_stream<RV, WV, true, false>), grid, block, 0, s, a, b, units, 0x9E3779B9u);          \
-        else if (nt_stores) hipLaunchKernelGGL((k_stream<RV, WV, false, true>), grid, block, 0, s, a, b, units, 0x9E3779B9u);         \
-        else hipLaunchKernelGGL((k_stream<RV, WV, false, false>), grid, block, 0, s, a, b, units, 0x9E3779B9u);                       \
+        if (nt_loads && nt_stores) hipLaunchKernelGGL((k_stream<RV, WV, true, true, STEPS>), grid, block, 0, s, a, b, units, 0x9E3779B9u);  \
+        else if (nt_loads) hipLaunchKernelGGL((k_stream<RV, WV, true, false, STEPS>), grid, block, 0, s, a, b, units, 0x9E3779B9u);          \
+        else if (nt_stores) hipLaunchKernelGGL((k_stream<RV, WV, false, true, STEPS>), grid, block, 0, s, a, b, units, 0x9E3779B9u);         \
+        else hipLaunchKernelGGL((k_stream<RV, WV, false, false, STEPS>), grid, block, 0, s, a, b, units, 0x9E3779B9u);                       \
     } while (0)
     switch (kind) {
     case C_RO: TFTQ_C(16, 0); break;
@@ -280,6 +286,10 @@ extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t
     case C_R4W1: TFTQ_C(16, 4); break;
     case C_R1W4: TFTQ_C(4, 16); break;
     case C_R8W1: TFTQ_C(16, 2); break;
+    case C_R2W1_4: TFTQ_CS(16, 8, 4); break;
+    case C_R1W2_4: TFTQ_CS(8, 16, 4); break;
+    case C_R4W1_4: TFTQ_CS(16, 4, 4); break;
+    case C_R1W4_4: TFTQ_CS(4, 16, 4); break;
     case C_RED:
     case C_RED_LINE: {
         if (row_bytes < 20 || row_bytes > 4100 || (row_bytes & 3) || rank < 0 || rank > 7) return -1;
