@@ -110,11 +110,8 @@ def cpu_baseline(fraction: float):
     except OSError:
         pass
     # For context: the same arithmetic written with torch CPU operators
-    # (tests/torch_restatement.py, the checker's cross-check), on 1/16 of the rows.
-    tests_dir = os.path.join(ROOT, "tests")
-    if tests_dir not in sys.path:
-        sys.path.insert(0, tests_dir)
-    import torch_restatement as trs
+    # (oracle/torch_restatement.py, the checker's cross-check), on 1/16 of the rows.
+    from oracle import torch_restatement as trs
     small = workloads.cfg3(0, scale_rows=1.0 / 16)
     small_ab = sum(workloads.algorithmic_bytes(small, ws).values())
     small_shapes = [tuple(t.shape) if t.dim() == 2 else (t.shape[0], 1) for t in small]

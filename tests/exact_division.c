@@ -6,6 +6,9 @@
  * run at e = 0; because every step scales exactly by powers of two while no
  * intermediate is subnormal, the boundary exponents e = -64 and e = +64 (the
  * ends of the range the kernels accept) are run too with the extreme codes.
+ * The kernels compute r_lo without the second divide, as one Newton step on
+ * e * r with e = fma(-s, r, 1):  lo = e * r,  r_lo = fma(fma(-s, lo, e), r, lo);
+ * the same loops check that this is RN(e / s) bit for bit.
  * Prints the number of mismatches; exit status 0 iff there are none.
  * Build: gcc -O2 -ffp-contract=off exact_division.c -lm
  */
@@ -30,7 +33,11 @@ int main(void)
         for (uint32_t man = 0; man < (1u << 23); man++) {
             const float s = u2f(((uint32_t)(127 + exps[ei]) << 23) | man);
             const float r = 1.0f / s;
-            const float r_lo = fmaf(-s, r, 1.0f) / s;
+            const float e = fmaf(-s, r, 1.0f);
+            const float r_lo = e / s;
+            const float lo = e * r;
+            if (fmaf(fmaf(-s, lo, e), r, lo) != r_lo) bad++;
+            total++;
             for (int i = 0; i < nf; i++) {
                 if (ei != 0 && i >= 8 && i < nf - 8) continue; /* extremes only */
                 const float f = fv[i];

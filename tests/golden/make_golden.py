@@ -1,7 +1,7 @@
 """Writes tests/golden/kat.json: known-answer vectors for the FP8 path.
 
 The vectors are computed here with torch's CPU float32 arithmetic and torch's
-own float8_e4m3fn cast (tests/torch_restatement.py), i.e. without the C checker
+own float8_e4m3fn cast (oracle/torch_restatement.py), i.e. without the C checker
 under oracle/ and without the HIP library, and were compared by hand with the
 closed forms: amax 4 -> scale 448/4 = 112 (0x42E00000); 1*112 = 112 -> 0x6E;
 -2*112 = -224 -> 0xF6; 0.5*112 = 56 -> 0x66; 4*112 = 448 -> 0x7E.
@@ -14,8 +14,8 @@ import sys
 
 import torch
 
-sys.path.insert(0, os.path.join(os.path.dirname(__file__), ".."))
-import torch_restatement as tr  # noqa: E402
+sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", ".."))
+from oracle import torch_restatement as tr  # noqa: E402
 
 
 def hexs(t: torch.Tensor) -> str:

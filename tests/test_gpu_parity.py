@@ -726,6 +726,13 @@ def test_cfg3_full_size(q, oracle):
     q.fused_reduce_fp8(list(peers_gpu[0]), recv, ws, rank, ReduceOp.AVG)
     oracle.fused_reduce_fp8(list(peer0_cpu), recv_cpu, ws, rank, ReduceOp.AVG, nthreads=NT)
     same_bytes(recv, recv_cpu, "cfg3 reduce rank 5")
+    # the configuration asks for SUM as well as AVG: another rank's slots, summed
+    recv_sum = sim.recv_buffer(qs, 2, ws)
+    recv_sum_cpu = recv_sum.cpu()
+    q.fused_reduce_fp8(list(peers_gpu[0]), recv_sum, ws, 2, ReduceOp.SUM)
+    oracle.fused_reduce_fp8(list(peer0_cpu), recv_sum_cpu, ws, 2, ReduceOp.SUM, nthreads=NT)
+    same_bytes(recv_sum, recv_sum_cpu, "cfg3 reduce rank 2, SUM")
+    del recv_sum, recv_sum_cpu
     # dequantize of that whole buffer (one reduced slot, seven as received), every tensor by bytes
     outs = [torch.empty_like(t) for t in peers_gpu[0]]
     outs_cpu = [torch.empty_like(t) for t in peer0_cpu]
@@ -927,11 +934,12 @@ def test_buffers_beyond_four_gib(q, oracle):
     assert torch.isfinite(outs[1][::4099].float()).all()
 
 
-def test_cfg5_full_size(q, oracle):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_cfg5_full_size(q, oracle, dtype):
     """All 10 000 ragged tensors, 16 peers, SUM: every peer's packed buffer, three
     ranks' reductions and the dequantized result against the checker."""
     shapes = workloads.cfg5_shapes(10000)
-    peers = [workloads.cfg5(s, torch.bfloat16, shapes) for s in range(16)]
+    peers = [workloads.cfg5(s, dtype, shapes) for s in range(16)]
     full_check(q, oracle, peers, 16, ReduceOp.SUM, ranks=[0, 9, 15])
     outs_g = [torch.empty_like(t).cuda() for t in peers[3]]
     outs_c = [torch.empty_like(t) for t in peers[3]]

@@ -225,3 +225,247 @@ def test_documented_binding(q, n_tensors):
         torch.cuda.synchronize()
         assert got.dtype == torch.uint8 and torch.equal(got, want)
     assert len(scope["_plans"]) == 1
+
+
+def _count_prepare(q, monkeypatch):
+    calls = []
+    real = q.prepare
+
+    def counting(*a, **k):
+        calls.append(1)
+        return real(*a, **k)
+
+    monkeypatch.setattr(q, "prepare", counting)
+    return calls
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_named_functions_recognise_a_long_list(q, oracle, monkeypatch, dtype):
+    """From the second call on, a list of more than 16 tensors that fits the plan of an
+    earlier call is checked and its addresses collected by one C++ walk: prepare() (the walk
+    in Python) is not called again, whatever tensors the list holds, and every call still
+    gives the checker's bytes."""
+    if q._pylist is None:
+        pytest.skip("torchft_amd._pylist is not built")
+    ws, rank, n = 4, 2, 40
+    lists = [make_list(n, 500 + p, dtype) for p in range(ws)]  # same shapes, other tensors and addresses
+    want = [oracle.fused_quantize_into_fp8([t.cpu() for t in ts], ws) for ts in lists]
+    same_bytes(q.fused_quantize_into_fp8(list(lists[0]), ws), want[0], "first call")
+    calls = _count_prepare(q, monkeypatch)
+    packed = [q.fused_quantize_into_fp8(list(ts), ws) for ts in lists]
+    packed += [q.fused_quantize_into_fp8(list(lists[1]), ws)]  # the addresses of two calls ago
+    assert not calls, "the Python walk ran for a list that fits a cached plan"
+    for k, (got, ref) in enumerate(zip(packed, want + [want[1]])):
+        same_bytes(got, ref, f"quantize of list {k}")
+
+    recv = sim.recv_buffer(packed[:ws], rank, ws)
+    ref = sim.recv_buffer(want, rank, ws)
+    for op in (ReduceOp.SUM, ReduceOp.AVG):
+        got_r, ref_r = recv.clone(), ref.clone()
+        q.fused_reduce_fp8(list(lists[0]), got_r, ws, rank, op)
+        oracle.fused_reduce_fp8([t.cpu() for t in lists[0]], ref_r, ws, rank, op)
+        same_bytes(got_r, ref_r, f"reduce {op}")
+
+    for k in (0, 3, 0):
+        outs = [torch.full_like(t, 7.0) for t in lists[k]]
+        outs_ref = [torch.empty_like(t.cpu()) for t in lists[k]]
+        q.fused_dequantize_from_fp8(outs, packed[k], ws)
+        oracle.fused_dequantize_from_fp8(outs_ref, want[k], ws)
+        for i, (a, b) in enumerate(zip(outs, outs_ref)):
+            same_bytes(a, b, f"dequantize of list {k}, tensor {i}")
+    assert not calls
+    with pytest.raises(AssertionError, match="Output size does not match"):
+        q.fused_dequantize_from_fp8(list(lists[0]), packed[0][:-4], ws)
+    with pytest.raises(AssertionError, match="Output size does not match"):
+        q.fused_reduce_fp8(list(lists[0]), packed[0][:-4], ws, rank)
+
+
+def test_long_list_whose_tensors_move_between_calls(q, oracle, monkeypatch):
+    """One list object, called again and again while its tensors change under it: storage
+    that moves (`.data =`), an element replaced by a tensor of the same shape, of another
+    shape, of another dtype, a 1-D element.  Every call sees the list as it is then."""
+    if q._pylist is None:
+        pytest.skip("torchft_amd._pylist is not built")
+    ws, n = 2, 24
+    ts = make_list(n, 900)
+
+    def check(what):
+        got = q.fused_quantize_into_fp8(ts, ws)
+        same_bytes(got, oracle.fused_quantize_into_fp8([t.cpu() for t in ts], ws), what)
+        return got
+
+    check("first call")
+    calls = _count_prepare(q, monkeypatch)
+    check("same list again")
+    old = ts[5]
+    ts[5].data = (old.float() * 3).to(old.dtype)  # new storage, same tensor object
+    assert ts[5] is old
+    check("a tensor whose storage moved")
+    ts[7] = (ts[7].float() - 1).to(ts[7].dtype)   # another tensor of the same shape
+    packed = check("an element replaced by another tensor")
+    assert not calls
+    outs = [torch.empty_like(t) for t in ts]
+    q.fused_dequantize_from_fp8(outs, packed, ws)
+    moved = [torch.empty_like(t) for t in ts]     # all outputs somewhere else, in one call
+    q.fused_dequantize_from_fp8(moved, packed, ws)
+    for i, (a, b) in enumerate(zip(outs, moved)):
+        same_bytes(a, b, f"dequantize into moved tensor {i}")
+    assert not calls
+    ts[3] = torch.randn(11, 77, device="cuda").to(ts[0].dtype)  # another shape: a new plan
+    check("an element of another shape")
+    assert len(calls) == 1
+    check("the new shapes again")
+    assert len(calls) == 1
+    ts[4] = ts[4].t().contiguous().t()            # same shape, other strides
+    check("an element with other strides")
+    assert len(calls) == 2
+    ts[6] = torch.randn(50, device="cuda").to(ts[0].dtype)      # 1-D: becomes [50, 1] in the list
+    check("a 1-D element")
+    assert ts[6].dim() == 2 and len(calls) == 3
+    check("after the 1-D element became 2-D")
+    assert len(calls) == 3
+    ts[2] = ts[2].float()
+    with pytest.raises(AssertionError, match="same dtype"):
+        q.fused_quantize_into_fp8(ts, ws)
+    ts[2] = ts[2].to(ts[0].dtype).cpu()
+    with pytest.raises(AssertionError, match="same device"):
+        q.fused_quantize_into_fp8(ts, ws)
+
+
+def test_long_list_on_several_streams_and_under_capture(q, oracle, monkeypatch):
+    """The address buffer of the fast path belongs to one device and stream: calls on other
+    streams, with other tensors, do not disturb each other; a call recorded by a stream
+    capture leaves nothing behind that a later call would trust."""
+    if q._pylist is None:
+        pytest.skip("torchft_amd._pylist is not built")
+    ws, n = 2, 30
+    a, b = make_list(n, 41), make_list(n, 42)
+    want_a = oracle.fused_quantize_into_fp8([t.cpu() for t in a], ws)
+    want_b = oracle.fused_quantize_into_fp8([t.cpu() for t in b], ws)
+    q.fused_quantize_into_fp8(list(a), ws)
+    torch.cuda.synchronize()
+    calls = _count_prepare(q, monkeypatch)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got = []
+    for rep in range(3):
+        with torch.cuda.stream(s1):
+            torch.cuda._sleep(int(5.0e7))
+            got.append((q.fused_quantize_into_fp8(list(a), ws), want_a))
+        with torch.cuda.stream(s2):
+            got.append((q.fused_quantize_into_fp8(list(b), ws), want_b))
+        got.append((q.fused_quantize_into_fp8(list(b if rep % 2 else a), ws), want_b if rep % 2 else want_a))
+    torch.cuda.synchronize()
+    for k, (g, w) in enumerate(got):
+        same_bytes(g, w, f"call {k}")
+    assert not calls
+
+    # a capture records the upload of b's addresses; the eager call after it must not take
+    # the buffer to hold them
+    cap = torch.cuda.Stream()
+    cap.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    out_b = [torch.empty_like(t) for t in b]
+    packed_b = q.fused_quantize_into_fp8(list(b), ws)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(cap):
+        q.fused_dequantize_from_fp8(list(a), q.fused_quantize_into_fp8(list(a), ws), ws)  # warm the stream's state
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=cap):
+            q.fused_dequantize_from_fp8(out_b, packed_b, ws)
+        out_b2 = [torch.empty_like(t) for t in b]
+        q.fused_dequantize_from_fp8(out_b2, packed_b, ws)  # eager, same stream, before any replay
+    torch.cuda.synchronize()
+    ref = [torch.empty_like(t.cpu()) for t in b]
+    oracle.fused_dequantize_from_fp8(ref, want_b, ws)
+    for i, (x, r) in enumerate(zip(out_b2, ref)):
+        same_bytes(x, r, f"eager call after the capture, tensor {i}")
+    for rep in range(2):
+        for t in out_b:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (x, r) in enumerate(zip(out_b, ref)):
+            same_bytes(x, r, f"replay {rep}, tensor {i}")
+
+
+def test_host_cost_of_the_named_functions_on_a_long_list(q):
+    """10 000 tensors through the three functions the reference names: after the first call
+    the host side of a call is a fraction of a millisecond."""
+    if q._pylist is None:
+        pytest.skip("torchft_amd._pylist is not built")
+    import workloads
+    shapes = workloads.cfg5_shapes(10000)
+    ts = workloads.cfg5(0, torch.bfloat16, shapes, device="cuda")
+    ws = 16
+    packed = q.fused_quantize_into_fp8(ts, ws)
+    want = q.prepare(ts, ws).quantize()
+    q.fused_reduce_fp8(ts, packed.clone(), ws, 3)
+    q.fused_dequantize_from_fp8(ts, packed, ws)
+    torch.cuda.synchronize()
+    n = 20
+    t0 = time.perf_counter()
+    for _ in range(n):
+        p = q.fused_quantize_into_fp8(ts, ws)
+        q.fused_reduce_fp8(ts, p, ws, 3, ReduceOp.SUM)
+        q.fused_dequantize_from_fp8(ts, packed, ws)
+    host_ms = (time.perf_counter() - t0) / n * 1e3
+    torch.cuda.synchronize()
+    print(f"{host_ms:.3f} ms of host time per quantize + reduce + dequantize on 10 000 tensors")
+    assert host_ms < 2.0, f"{host_ms:.2f} ms of host time per step through the named functions"
+    same_bytes(q.fused_quantize_into_fp8(ts, ws), want, "10 000 tensors")
+
+
+@pytest.mark.parametrize("n_tensors", [1, 5, 30])
+def test_prepared_bucket_is_bound_to_its_tensors(q, n_tensors):
+    """`prepared=` of allreduce_quantized must be the bucket of these very tensors: a bucket of
+    other tensors, or of tensors that have moved since, is refused instead of reducing the
+    old addresses."""
+    from torchft_amd import collectives as col
+    ws = 2
+    ts = make_list(n_tensors, 77)
+    bucket = q.prepare(ts, ws)
+    assert bucket.matches(ts) and bucket.matches(list(ts)) and bucket.matches(tuple(ts))
+    flat = torch.randn(1000, device="cuda")
+    one = q.prepare([flat], ws)            # the bucket holds the [1000, 1] view
+    assert one.matches([flat]) and one.matches([flat.unsqueeze(1)]) and not one.matches([flat.clone()])
+    assert not one.matches([flat[::2]]) and not one.matches([flat.double()])
+    others = make_list(n_tensors, 77)      # same values and shapes, other addresses
+    assert not bucket.matches(others) and not bucket.matches(ts[:-1]) and not bucket.matches(ts + ts[:1])
+    group = SimGroup(1)
+    with pytest.raises(ValueError, match="prepare again"):
+        col.allreduce_quantized(others, ReduceOp.SUM, group.rank(0), prepared=bucket)
+    moved = list(ts)
+    moved[0].data = moved[0].clone()
+    assert not bucket.matches(moved)
+    with pytest.raises(ValueError, match="prepare again"):
+        col.allreduce_quantized(moved, ReduceOp.SUM, group.rank(0), prepared=bucket)
+    with pytest.raises(ValueError, match="prepare again"):
+        col.allreduce_quantized(ts, ReduceOp.SUM, group.rank(0), prepared=q.prepare(ts, 4))
+
+
+def test_first_use_of_a_bucket_under_capture(q):
+    """A bucket of a long list whose first compute call is recorded by a stream capture: the
+    capture holds the upload of the addresses, and eager calls after it, on this stream and
+    on another, upload them themselves instead of trusting an upload that has not run."""
+    ws = 2
+    ts = make_list(30, 5)
+    want = q.prepare(make_list(30, 5), ws).quantize()
+    torch.cuda.synchronize()
+    bucket = q.prepare(ts, ws)
+    out = torch.empty(bucket.output_size, dtype=torch.uint8, device="cuda")
+    cap = torch.cuda.Stream()
+    cap.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(cap):
+        with torch.cuda.graph(graph, stream=cap):
+            bucket.quantize(out=out)
+        eager_same = bucket.quantize()
+    eager_default = bucket.quantize()
+    torch.cuda.synchronize()
+    same_bytes(eager_same, want, "eager call on the capture's stream")
+    same_bytes(eager_default, want, "eager call on the default stream")
+    for rep in range(2):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        same_bytes(out, want, f"replay {rep}")

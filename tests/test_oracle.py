@@ -10,7 +10,7 @@ What pins what:
   f16 / bf16  numpy float16 and torch bfloat16 casts
   Q / R / D   golden vectors in tests/golden/kat.json (hand-checked closed
               forms); byte equality with the independent torch restatement
-              (tests/torch_restatement.py) on random, odd, strided inputs; a
+              (oracle/torch_restatement.py) on random, odd, strided inputs; a
               straight-line numpy-float32 brute force on tiny inputs;
               mathematical special cases (ws = 1 SUM is the identity on codes,
               identical peers with power-of-two ws average back to the input
@@ -26,7 +26,7 @@ import pytest
 import torch
 from torch.distributed import ReduceOp
 
-import torch_restatement as tr
+from oracle import torch_restatement as tr
 import workloads
 
 HERE = os.path.dirname(os.path.abspath(__file__))

@@ -17,6 +17,9 @@ SOURCES = ["tftq_quantize.hip", "tftq_reduce.hip", "tftq_dequantize.hip", "tftq_
 # (benchmark infrastructure; torchft_amd never loads this library).
 CEILING_LIB_PATH = os.path.join(_HERE, "libtftq_ceiling.so")
 CEILING_SOURCE = "tftq_ceiling.hip"
+# The C++ walk over lists of tensors: a CPython extension module built with the host compiler
+# against the Python and libtorch headers.  Host code only; not part of libtftq.so.
+PYLIST_SOURCE = "tftq_pylist.cpp"
 
 # -ffp-contract=off: the arithmetic contract is separate IEEE multiply, divide
 # and add; fused multiply-adds are written out where they are wanted.
@@ -34,7 +37,7 @@ def source_hash() -> str:
     built with as tftq_build_id()."""
     h = hashlib.sha256()
     files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC))
-             if f.endswith((".hip", ".h", ".cpp")) and f != CEILING_SOURCE]
+             if f.endswith((".hip", ".h", ".cpp")) and f not in (CEILING_SOURCE, PYLIST_SOURCE)]
     files.append(os.path.join(os.path.dirname(_HERE), "include", "tftq.h"))
     for path in files:
         h.update(os.path.basename(path).encode() + b"\0")
@@ -48,6 +51,68 @@ def hipcc_path() -> str:
         if cand and os.path.exists(cand):
             return cand
     raise RuntimeError("hipcc not found; libtftq.so cannot be built")
+
+
+# The C++ walk over lists of tensors (tftq_pylist.cpp): a CPython extension module built with
+# the host compiler against the Python and libtorch headers.  Host code only.
+
+
+
+def pylist_path() -> str:
+    import sysconfig
+    return os.path.join(_HERE, "_pylist" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+
+def pylist_hash() -> str:
+    with open(os.path.join(CSRC, PYLIST_SOURCE), "rb") as fh:
+        return hashlib.sha256(fh.read()).hexdigest()[:16]
+
+
+def pylist_command() -> list[str]:
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("no C++ compiler found; _pylist cannot be built")
+    libdir = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f'-DTFTQ_PYLIST_ID="{pylist_hash()}"']
+    cmd += ["-I" + d for d in cpp_extension.include_paths()]
+    cmd += ["-I" + sysconfig.get_paths()["include"], "-o", pylist_path(), os.path.join(CSRC, PYLIST_SOURCE),
+            "-L" + libdir, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10", "-Wl,-rpath," + libdir]
+    return cmd
+
+
+def build_pylist() -> str:
+    _run(pylist_command())
+    return pylist_path()
+
+
+def load_pylist():
+    """The _pylist module, built first if there is no build or if the build is of another
+    source; None (with a warning) when it can be neither loaded nor built.  Callers then
+    walk their lists in Python: same results, more host time on long lists."""
+    import importlib
+    import warnings
+    for attempt in (0, 1):
+        try:
+            if attempt == 1 or not os.path.exists(pylist_path()):
+                build_pylist()
+            mod = importlib.import_module("torchft_amd._pylist")
+            if getattr(mod, "BUILD_ID", None) == pylist_hash() or os.environ.get("TFTQ_ALLOW_STALE"):
+                return mod
+            if attempt == 1:  # a module that is already imported cannot be replaced in this process
+                warnings.warn("torchft_amd._pylist was built from another source; rebuild it with "
+                              "`python -m torchft_amd._build` (lists are walked in Python until then)")
+                return None
+        except Exception as exc:  # missing compiler or headers, an ABI that does not load
+            if attempt == 1:
+                warnings.warn(f"torchft_amd._pylist is not available ({exc}); lists are walked in Python")
+                return None
+    return None
 
 
 def _run(cmd: list[str]) -> str:
@@ -68,6 +133,7 @@ def build_library(verbose: bool = False) -> str:
         build_id = f'-DTFTQ_BUILD_ID="{source_hash()}"'
         cmds = [[hipcc, *HIPCC_FLAGS, build_id, "-c", "-o", o, os.path.join(CSRC, s)] for s, o in zip(SOURCES, objs)]
         cmds.append([hipcc, *HIPCC_FLAGS, "-shared", "-o", CEILING_LIB_PATH, os.path.join(CSRC, CEILING_SOURCE)])
+        cmds.append(pylist_command())
         with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
             outs = list(pool.map(_run, cmds))
         outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]))

@@ -207,8 +207,11 @@ def allreduce_quantized(
     ex = _begin(opts, AllreduceOptions, "allreduce", process_group, sync_stream)
     ws, rank = ex.world_size, ex.rank
 
-    if prepared is not None and (prepared.ws != ws or len(prepared.tensors) != len(tensors)):
-        raise ValueError("`prepared` was made for another tensor list or group size")
+    # the bucket's kernels read and write the addresses bound by prepare(): tensors that are not
+    # those, or have moved since, would be left untouched without a word
+    if prepared is not None and (prepared.ws != ws or not prepared.matches(tensors)):
+        raise ValueError("`prepared` was made for another group size or for other tensors than these "
+                         "(other shapes, strides, dtype, device, or storage that has moved since): prepare again")
 
     with cuda.stream(ex.stream):
         # one walk over the list for all three kernels; the bucket holds the tensors, so the

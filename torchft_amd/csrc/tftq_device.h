@@ -154,12 +154,18 @@ struct DivCoef {
 // positive, exponent in [-64, 64]
 DEV bool scale_is_fast(float s) { return (as_u(s) - (63u << 23)) < (129u << 23); }
 
+// r_lo = RN(e / s) with e = fma(-s, r, 1), without a second divide: one Newton step on
+// e * r gives the correctly rounded quotient for every scale in the fast range
+// (tests/exact_division.c compares the two for all 2^23 mantissas); outside that range
+// the coefficients are not used.
 DEV DivCoef make_div(float s)
 {
     DivCoef c;
     c.s = s;
     c.r = 1.0f / s;
-    c.r_lo = __builtin_fmaf(-s, c.r, 1.0f) / s;
+    const float e = __builtin_fmaf(-s, c.r, 1.0f);
+    const float lo = e * c.r;
+    c.r_lo = __builtin_fmaf(__builtin_fmaf(-s, lo, e), c.r, lo);
     c.fast = scale_is_fast(s);
     return c;
 }
@@ -354,7 +360,6 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
     const int x = (int)(blockIdx.x & 7);
     int i = (int)(blockIdx.x >> 3);
     if (INLINE) {
-        if (p.natural) i = (int)blockIdx.x;  // all eight rows of the table describe the whole work
         // One round of scalar loads fetches this XCD's three table rows; the position
         // is then found in registers, and only the segment descriptor needs a second round.
         const CONSTANT char *karg = (const CONSTANT char *)__builtin_amdgcn_kernarg_segment_ptr();
@@ -365,7 +370,9 @@ DEV bool locate(const KParams &p, const InlineTable &inl, Seg &s, int &vb)
         const Row seg = *(const CONSTANT Row *)(d + offsetof(Dealt, seg) / 4);
         Row cum_end_ = cum_end, base_ = base, seg_ = seg;
         // all scalar loads of this round, and the common parameters, are issued before the first wait
-        asm volatile("" : "+s"(cum_end_), "+s"(base_), "+s"(seg_) : "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
+        int natural = p.natural;
+        asm volatile("" : "+s"(cum_end_), "+s"(base_), "+s"(seg_), "+s"(natural) : "s"(p.packed), "s"(p.slot_size), "s"(p.ws), "s"(p.rank));
+        if (natural) i = (int)blockIdx.x;  // all eight rows of the table describe the whole work
         int b = base_[0], sg = seg_[0];
 #pragma unroll
         for (int j = 1; j < TFTQ_N_INLINE; j++) {

@@ -67,7 +67,12 @@ DEV void store_codes(GLOBAL u32 *payload, int d0, int ndw, const u32x4 w)
     }
 }
 
-// acc[e] += code[e] / s for the 16 codes of w, s given as (r, r_lo)
+// acc[e] += code[e] / s for the 16 codes of w, s given as (r, r_lo).
+// FIRST: acc[e] = code[e] / s, for the first peer of a row.  The reference starts from
+// zeros (:405) and 0 + q is q for every q but -0, so the sums can only differ when every
+// peer contributes -0: then this sum is -0 where the reference has +0.  requant16 makes
+// up for that (a negative zero sum is encoded as +0); the row maximum does not see it.
+template <bool FIRST = false>
 DEV void accumulate16(float (&acc)[16], const u32x4 w, float r, float r_lo)
 {
     const u32 ww[4] = {w.x, w.y, w.z, w.w};
@@ -77,7 +82,10 @@ DEV void accumulate16(float (&acc)[16], const u32x4 w, float r, float r_lo)
         float f[4];
         unpack_fp8x4(ww[t], f);
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc[4 * t + e] = acc[4 * t + e] + div_fast(f[e], r, r_lo);
+        for (int e = 0; e < 4; e++) {
+            const float q = div_fast(f[e], r, r_lo);
+            acc[4 * t + e] = FIRST ? q : acc[4 * t + e] + q;
+        }
     }
 }
 
@@ -95,7 +103,7 @@ DEV void accumulate16(float (&acc)[16], const u32x4 w, float r, float r_lo)
 template <bool GDIV, bool IEEE = false>
 DEV float scale_div(float a, float s2, const KParams &p)
 {
-    const float y = a * s2;
+    const float y = __builtin_fmaf(a, s2, 0.0f);  // a * s2, and +0 for a sum of -0 (see accumulate16)
     if (!GDIV) return y * p.inv_div;
     if (IEEE) return y / p.div;
     const float q0 = y * p.inv_div;
@@ -122,7 +130,7 @@ DEV u32x4 requant16(const float (&a)[16], float s2, const KParams &p)
     const bool fold = !GDIV && (sf == 0.0f || __builtin_fabsf(sf) >= 1.17549435e-38f);
     if (__builtin_amdgcn_ballot_w64(!fold) == 0) {  // one code path per wavefront
 #pragma unroll
-        for (int e = 0; e < 16; e++) y[e] = a[e] * sf;
+        for (int e = 0; e < 16; e++) y[e] = __builtin_fmaf(a[e], sf, 0.0f);  // a * sf, and +0 for a sum of -0
     } else {
 #pragma unroll
         for (int e = 0; e < 16; e++) y[e] = scale_div<GDIV>(a[e], s2, p);
@@ -450,12 +458,14 @@ DEV void reduce_row(const Seg &s, const KParams &p, int j, int lane, float *lds)
 // row length: independent workgroups keep more loads in flight.)
 constexpr int R_VPB = 4;
 
-template <int TEAM, int UNITS, bool PIPE, bool GDIV>
+template <int TEAM, int UNITS, bool PIPE, bool GDIV, int WS = 0>
 DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds, bool valid = true)
 {
     constexpr int PB = R_VPB / UNITS >= 1 ? R_VPB / UNITS : 1;  // peers per batch
     const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
-    const int ws = p.ws;
+    // WS: the group size when it is known at compile time (the loops over the peers then
+    // unroll into straight-line code); 0: p.ws
+    const int ws = WS ? WS : p.ws;
     const int nb = (ws + PB - 1) / PB;  // batches
     const int wlane = TEAM >= 64 ? (int)(threadIdx.x & 63u) : lane;
     const int speer = min(wlane, ws - 1);  // the peer whose scale this lane fetches
@@ -490,80 +500,84 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
         }
     };
 
-    float acc[UNITS][16];
+    issue(A, 0);
+    if (PIPE && nb > 1) issue(B, 1);
+    // the loads above are issued before anything below: left to itself, the scheduler moves
+    // them down between the accumulation steps of the straight-line variants
+    __builtin_amdgcn_sched_barrier(0);
+
+    const float sc = raw_scale == 0.0f ? 1.0f : raw_scale;  // padding rows (:419)
+    const DivCoef c = make_div(sc);
+    if (__builtin_amdgcn_ballot_w64(!c.fast) != 0) {  // same in all wavefronts of the team
+        if (valid) reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
+        return;
+    }
+
+    float acc[UNITS][16];  // set by the first peer
+    auto consume = [&](const Batch &src, int batch, auto first_c) {
+        constexpr bool FIRST = decltype(first_c)::value;
+#pragma unroll
+        for (int b = 0; b < PB; b++) {
+            const int k = batch * PB + b;
+            if (k < ws) {
+                const float pr = team_bcast<TEAM>(c.r, k), pl = team_bcast<TEAM>(c.r_lo, k);
+#pragma unroll
+                for (int u = 0; u < UNITS; u++) {
+                    u32x4 w = src.w[b][u];
+                    w.w &= padmask[u];  // here, not at the load: the load must stay in flight
+                    if (FIRST && b == 0) accumulate16<true>(acc[u], w, pr, pl);
+                    else accumulate16<false>(acc[u], w, pr, pl);
+                }
+            }
+            // peer after peer: work of later peers that is moved up here only holds registers
+            if (WS) __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    const std::true_type first;
+    const std::false_type later;
+
+    consume(A, 0, first);
+    if (!PIPE) {  // long rows: one batch in flight keeps the register count down
+#pragma nounroll
+        for (int i = 1; i < nb; i++) {
+            issue(A, i);
+            consume(A, i, later);
+        }
+    } else if (WS) {  // straight-line code: batch i in B for odd i, in A for even i
+#pragma unroll
+        for (int i = 1; i < (WS + PB - 1) / PB; i++) {
+            if (i + 1 < (WS + PB - 1) / PB) {
+                issue((i & 1) ? A : B, i + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            consume((i & 1) ? B : A, i, later);
+        }
+    } else {
+#pragma nounroll
+        for (int i = 1; i < nb; i += 2) {  // B holds batch i
+            if (i + 1 < nb) issue(A, i + 1);
+            consume(B, i, later);
+            if (i + 1 < nb) {
+                if (i + 2 < nb) issue(B, i + 2);
+                consume(A, i + 1, later);
+            }
+        }
+    }
+
+    float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
 #pragma unroll
     for (int u = 0; u < UNITS; u++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
-    float cr = 1.0f, cl = 0.0f;
-    bool row_fast = true;
-
-    auto consume = [&](const Batch &src, int batch) {
-        if (batch == 0) {
-            const float sc = raw_scale == 0.0f ? 1.0f : raw_scale;  // padding rows (:419)
-            const DivCoef c = make_div(sc);
-            cr = c.r;
-            cl = c.r_lo;
-            row_fast = __builtin_amdgcn_ballot_w64(!c.fast) == 0;  // same in all wavefronts of the team
-        }
-        if (row_fast) {
+        for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+    amax = team_max<TEAM>(amax, lds);
+    const float s2 = calc_scale(amax_div<GDIV>(amax, p));  // :340
+    GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
 #pragma unroll
-            for (int b = 0; b < PB; b++) {
-                const int k = batch * PB + b;
-                if (k < ws) {
-                    const float pr = team_bcast<TEAM>(cr, k), pl = team_bcast<TEAM>(cl, k);
-#pragma unroll
-                    for (int u = 0; u < UNITS; u++) {
-                        u32x4 w = src.w[b][u];
-                        w.w &= padmask[u];  // here, not at the load: the load must stay in flight
-                        accumulate16(acc[u], w, pr, pl);
-                    }
-                }
-            }
-        }
-    };
-
-    if (!PIPE) {  // long rows: one batch in flight keeps the register count down
-        for (int i = 0; i < nb; i++) {
-            issue(A, i);
-            consume(A, i);
-        }
-    } else {
-        issue(A, 0);
-        int i = 0;
-        for (; i + 2 < nb; i += 2) {
-            issue(B, i + 1);
-            consume(A, i);
-            issue(A, i + 2);
-            consume(B, i + 1);
-        }
-        if (i + 1 < nb) {
-            issue(B, i + 1);
-            consume(A, i);
-            consume(B, i + 1);
-        } else {
-            consume(A, i);
-        }
+    for (int u = 0; u < UNITS; u++) {
+        const u32x4 o = requant16<GDIV>(acc[u], s2, p);
+        if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
     }
-
-    if (row_fast) {
-        float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
-#pragma unroll
-        for (int u = 0; u < UNITS; u++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
-        amax = team_max<TEAM>(amax, lds);
-        const float s2 = calc_scale(amax_div<GDIV>(amax, p));  // :340
-        GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
-#pragma unroll
-        for (int u = 0; u < UNITS; u++) {
-            const u32x4 o = requant16<GDIV>(acc[u], s2, p);
-            if (valid && 4 * (u * TEAM + lane) < ndw) *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = o;
-        }
-        if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
-    } else if (valid) {
-        reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
-    }
+    if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
 }
 
 // One row per team with UNITS >= 2 vectors per lane and peer, as a rolling window over the
@@ -788,6 +802,15 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
     }
 }
 
+// reduce_rows for a team of TEAM lanes with UNITS vectors per lane and peer: groups of 8 and
+// of 4 peers run straight-line code (averages over such groups never need GDIV)
+#define TFTQ_REDUCE_ROWS(TEAM, UNITS, ...)                                                        \
+    do {                                                                                          \
+        if (!GDIV && p.ws == 8) reduce_rows<TEAM, UNITS, true, GDIV, GDIV ? 0 : 8>(__VA_ARGS__);  \
+        else if (!GDIV && p.ws == 4) reduce_rows<TEAM, UNITS, true, GDIV, GDIV ? 0 : 4>(__VA_ARGS__); \
+        else reduce_rows<TEAM, UNITS, true, GDIV>(__VA_ARGS__);                                   \
+    } while (0)
+
 template <bool INLINE, bool GDIV, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams p, const InlineTable inl)
 {
@@ -864,12 +887,12 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
             const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
             // (at least one: a wavefront past the end of a short row still takes part in the barriers)
             const int nu = max(1, min((ndw + 1023) >> 10, (ndw - 256 * wave + 1023) >> 10));
-            if (nu == 1) reduce_rows<256, 1, true, GDIV>(s, p, j, tid, lds);
+            if (nu == 1) TFTQ_REDUCE_ROWS(256, 1, s, p, j, tid, lds);
             // rows of three or four vectors per lane run the rolling window in all their wavefronts
             // ([20480, 10240]: 53.5 -> 50.4 us against the pipeline in the upper two); rows of two
             // are faster in the pipeline (5120 columns: 50.9 against 62.1 us)
             else if (nu == 2 && ndw > 2048) reduce_rows_roll<256, 2, GDIV>(s, p, j, tid, lds);
-            else if (nu == 2) reduce_rows<256, 2, true, GDIV>(s, p, j, tid, lds);
+            else if (nu == 2) TFTQ_REDUCE_ROWS(256, 2, s, p, j, tid, lds);
             else if (nu == 3) reduce_rows_roll<256, 3, GDIV>(s, p, j, tid, lds);
             else reduce_rows_roll<256, 4, GDIV>(s, p, j, tid, lds);
         }
@@ -889,9 +912,9 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
             else if (ndw <= 512) reduce_row<64, 2, GDIV>(s, p, j, tid & 63, lds);
             else reduce_row_slow<64, GDIV>(s, p, j, tid & 63, lds);
         } else if (ndw <= 256) {
-            reduce_rows<64, 1, true, GDIV>(s, p, j, tid & 63, lds);
+            TFTQ_REDUCE_ROWS(64, 1, s, p, j, tid & 63, lds);
         } else if (ndw <= 512) {
-            reduce_rows<64, 2, true, GDIV>(s, p, j, tid & 63, lds);
+            TFTQ_REDUCE_ROWS(64, 2, s, p, j, tid & 63, lds);
         } else {
             reduce_rows_roll<64, 3, GDIV>(s, p, j, tid & 63, lds);
         }

@@ -23,6 +23,14 @@ list once and returns a :class:`PreparedBucket` whose ``quantize`` / ``reduce`` 
 ``dequantize`` cost the same few microseconds whatever the length of the list:
 the thing to hold on to for a bucket that is reduced every step.
 
+Lists of more than 16 tensors that come back call after call (the same shapes,
+strides, dtype and device; the tensors themselves may be new or may have moved)
+are recognised by one C++ walk over the list (``_pylist.scan``, about 10 ns per
+tensor), which checks every tensor against the plan of an earlier call and
+collects the addresses; the three functions then cost a fraction of a
+millisecond on 10 000 tensors instead of the 5 ms of the walk in Python, which
+stays as the path of every first call and of every list that does not match.
+
 There is no CPU or eager fallback: without the HIP library and a gfx950 device
 the functions raise.
 """
@@ -39,7 +47,9 @@ from collections import OrderedDict
 import torch
 from torch.distributed import ReduceOp
 
-from . import _lib
+from . import _build, _lib
+
+_pylist = _build.load_pylist()  # None when the helper cannot be built: the Python walk does everything
 
 SCALE_DTYPE: torch.dtype = torch.float32
 SCALE_DTYPE_BYTES: int = 4
@@ -69,7 +79,9 @@ class _Ready:
         ev = self.event
         if ev is None or raw_stream == self.stream_id:  # done, or ordered by the stream itself
             return
-        if ev.query():
+        if torch.cuda.is_current_stream_capturing():
+            stream.wait_event(ev)  # a capture may wait for an outside event, but not ask about it
+        elif ev.query():
             self.event = None
         else:
             stream.wait_event(ev)
@@ -80,12 +92,22 @@ class _Plan:
     device it has been used on.  Holds no tensor and no address."""
 
     __slots__ = ("handle", "output_size", "slot_size", "max_rows", "n_tensors", "table_bytes",
-                 "tables", "_lib", "_lock")
+                 "tables", "_lib", "_lock", "dtype_code", "ws", "shapes", "strides", "a_shapes",
+                 "a_strides", "streams")
 
-    def __init__(self, lib, handle, n_tensors):
+    def __init__(self, lib, handle, n_tensors, dtype_code, ws, shapes, strides):
         self._lib = lib
         self.handle = handle
         self.n_tensors = n_tensors
+        self.dtype_code = dtype_code
+        self.ws = ws
+        # what the plan was built from, [n_tensors][2] int64 each: _pylist.scan compares a list with them
+        self.shapes = shapes
+        self.strides = strides
+        self.a_shapes = ctypes.addressof(shapes)
+        self.a_strides = ctypes.addressof(strides)
+        # long lists through the named functions: (device index, raw stream) -> _StreamPointers
+        self.streams: "OrderedDict[tuple, _StreamPointers]" = OrderedDict()
         self.output_size = lib.tftq_plan_output_size(handle)
         self.slot_size = lib.tftq_plan_slot_size(handle)
         self.max_rows = lib.tftq_plan_max_rows(handle)
@@ -175,19 +197,124 @@ def _plan_for(dtype: torch.dtype, ws: int, sizes_key: tuple, strides_key: tuple)
     handle = ctypes.c_void_p()
     _check(lib.tftq_plan_create(_DTYPE_CODE[dtype], T, shapes, strides, ws, ctypes.byref(handle)),
            "tftq_plan_create")
-    plan = _Plan(lib, handle, T)
+    plan = _Plan(lib, handle, T, _DTYPE_CODE[dtype], ws, shapes, strides)
     global _plan_cache_tensors
     with _cache_lock:
         old = _plan_cache.pop(key, None)  # another thread may have built the same plan
         if old is not None:
             _plan_cache_tensors -= old.n_tensors
+            _forget_long_plan(old)
         _plan_cache[key] = plan
         _plan_cache_tensors += T
+        if T > _N_INLINE:
+            _long_plans.setdefault((T, ws), []).insert(0, plan)
         while len(_plan_cache) > 1 and (len(_plan_cache) > _PLAN_CACHE_SIZE
                                         or _plan_cache_tensors > _PLAN_CACHE_TENSORS):
             _, gone = _plan_cache.popitem(last=False)
             _plan_cache_tensors -= gone.n_tensors
+            _forget_long_plan(gone)
     return plan
+
+
+# ---------------------------------------------------------------------------------------------
+# long lists through the three named functions
+# ---------------------------------------------------------------------------------------------
+# Plans of more than 16 tensors by (number of tensors, group size), newest first: the plans a
+# list of that length is compared with by _pylist.scan before the Python walk is tried.
+_long_plans: "dict[tuple, list[_Plan]]" = {}
+_LONG_CANDIDATES = 4    # plans of one length and group size that a call compares its list with
+_STREAMS_PER_PLAN = 8   # address buffers (one per device and stream) that a plan keeps
+
+
+def _forget_long_plan(plan: _Plan) -> None:  # called with _cache_lock held
+    peers = _long_plans.get((plan.n_tensors, plan.ws))
+    if peers is not None and plan in peers:
+        peers.remove(plan)
+        if not peers:
+            del _long_plans[(plan.n_tensors, plan.ws)]
+
+
+class _StreamPointers:
+    """What a plan keeps for calls on one stream of one device: the device copy of a long
+    list's addresses and what it holds, so that a call whose list has the addresses of the
+    last one uploads nothing."""
+
+    __slots__ = ("dev", "held", "lock")
+
+    def __init__(self, plan: _Plan, device: torch.device, table: torch.Tensor) -> None:
+        with torch.cuda.device(device):
+            stream = torch.cuda.current_stream(device)
+            self.dev = torch.empty(plan.n_tensors, dtype=torch.int64, device=device)
+            # both are read by kernels on this stream, which need not be the one they were allocated on
+            self.dev.record_stream(stream)
+            table.record_stream(stream)
+        self.held = None   # host array of the addresses that `dev` holds (or will, in stream order)
+        self.lock = threading.Lock()
+
+
+_memcmp = ctypes.CDLL(None).memcmp
+_memcmp.restype = ctypes.c_int
+_memcmp.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+
+
+def _match_long_list(inputs, ws: int, want_pointers: bool):
+    """(plan, device, addresses) when `inputs` is a list of more than 16 tensors that fits a
+    plan of an earlier call as it is (same length, group size, dtype, sizes and strides, every
+    tensor 2-D and on one GPU), found with one C++ walk per candidate plan; else None, and
+    the caller takes the Python walk.  addresses: a fresh host array, or None when not wanted."""
+    if _pylist is None or type(inputs) is not list:
+        return None
+    T = len(inputs)
+    if T <= _N_INLINE:
+        return None
+    peers = _long_plans.get((T, ws))
+    if not peers:
+        return None
+    first = inputs[0]
+    if not isinstance(first, _TENSOR):
+        return None
+    device = first.device
+    if device.type != "cuda":
+        return None
+    ptrs = (ctypes.c_void_p * T)() if want_pointers else None
+    a_ptrs = ctypes.addressof(ptrs) if want_pointers else 0
+    for plan in peers[:_LONG_CANDIDATES]:
+        if _pylist.scan(inputs, plan.dtype_code, device.index, plan.a_shapes, plan.a_strides, a_ptrs, T) == T:
+            return plan, device, ptrs
+    return None
+
+
+def _long_list_args(plan: _Plan, device: torch.device, raw_stream: int, ptrs):
+    """(table, pointers, lock to hold until the kernel is queued) for a compute call on a
+    matched long list.  The addresses are uploaded on the call's stream unless the buffer
+    of this device and stream holds them already (ptrs None: no addresses wanted, no lock)."""
+    table, ready = plan.table_on(device)
+    if ready.event is not None:
+        ready.wait(torch.cuda.current_stream(device), raw_stream)
+    key = (device.index, raw_stream)
+    sp = plan.streams.get(key)
+    if sp is None:
+        with plan._lock:
+            sp = plan.streams.get(key)
+            if sp is None:
+                sp = _StreamPointers(plan, device, table)
+                plan.streams[key] = sp
+                while len(plan.streams) > _STREAMS_PER_PLAN:
+                    plan.streams.popitem(last=False)
+    if ptrs is None:
+        return table.data_ptr(), None, None
+    sp.lock.acquire()
+    try:
+        capturing = torch.cuda.is_current_stream_capturing()
+        if capturing or sp.held is None or _memcmp(sp.held, ptrs, 8 * plan.n_tensors) != 0:
+            _check(plan._lib.tftq_upload_pointers(plan.handle, ptrs, sp.dev.data_ptr(), device.index, raw_stream),
+                   "tftq_upload_pointers")
+            # an upload that a stream capture records has not run: the next call uploads again
+            sp.held = None if capturing else ptrs
+    except BaseException:
+        sp.lock.release()
+        raise
+    return table.data_ptr(), sp.dev.data_ptr(), sp.lock
 
 
 # Per-call host cost matters for the per-parameter all-reduce (thousands of small
@@ -251,6 +378,34 @@ class PreparedBucket:
     def slot_size(self) -> int:
         return self.plan.slot_size
 
+    def matches(self, tensors) -> bool:
+        """True when ``tensors`` are what this bucket was prepared for: as many tensors, of the
+        plan's dtype, sizes and strides (a 1-D tensor of k elements counts as ``[k, 1]``,
+        quantization.py:487-488), on the bucket's device, at the addresses the bucket has bound."""
+        plan = self.plan
+        n = plan.n_tensors
+        if len(tensors) != n:
+            return False
+        if _pylist is not None and type(tensors) is list:
+            got = (ctypes.c_void_p * n)()
+            if _pylist.scan(tensors, plan.dtype_code, self._dev_index, plan.a_shapes, plan.a_strides,
+                            ctypes.addressof(got), n) == n:
+                return _memcmp(got, self._ptrs, 8 * n) == 0
+        shapes, strides, ptrs = plan.shapes, plan.strides, self._ptrs
+        for i, t in enumerate(tensors):
+            if not isinstance(t, _TENSOR) or _DTYPE_CODE.get(t.dtype) != plan.dtype_code or t.device != self.device:
+                return False
+            if t.dim() == 2:
+                size, stride = tuple(t.shape), t.stride()
+            elif t.dim() == 1:
+                size, stride = (t.shape[0], 1), (t.stride(0), 1)
+            else:
+                return False
+            if (size[0] != shapes[2 * i] or size[1] != shapes[2 * i + 1] or stride[0] != strides[2 * i]
+                    or stride[1] != strides[2 * i + 1] or t.data_ptr() != (ptrs[i] or 0)):
+                return False
+        return True
+
     # -- launches ------------------------------------------------------------------------
     def _long_list_args(self, raw_stream: int, needs_pointers: bool):
         """(table, pointers) arguments of a compute call on a long list, both current for
@@ -269,7 +424,11 @@ class PreparedBucket:
                     # the first call on this bucket writes the addresses; later calls reuse them
                     _check(self._lib.tftq_upload_pointers(self._handle, self._ptrs, self._ptrs_dev.data_ptr(),
                                                           self._dev_index, raw_stream), "tftq_upload_pointers")
-                    self._ptrs_ready = _Ready(stream)
+                    # Under a stream capture the upload has only been recorded (it runs with the
+                    # graph, before the kernel recorded behind it): nothing is ready, and the
+                    # next call uploads again.
+                    if not torch.cuda.is_current_stream_capturing():
+                        self._ptrs_ready = _Ready(stream)
                     return self._table.data_ptr(), self._ptrs_dev.data_ptr()
         ready.wait(stream, raw_stream)
         return self._table.data_ptr(), self._ptrs_dev.data_ptr()
@@ -318,13 +477,16 @@ class PreparedBucket:
             _check(self._lib.tftq_dequantize(self._handle, tensors, table, pointers, packed.data_ptr(),
                                              plan.output_size, self._dev_index, raw), "tftq_dequantize")
         else:
-            # torch divides a GPU tensor by a host scalar as a multiplication by the
-            # reciprocal, computed in double and rounded to fp32
-            divisor = float(divide_by)
-            factor = 1.0 / divisor if divisor != 0.0 else math.copysign(math.inf, divisor)
             _check(self._lib.tftq_dequantize_scaled(self._handle, tensors, table, pointers, packed.data_ptr(),
-                                                    plan.output_size, factor, self._dev_index, raw),
+                                                    plan.output_size, _post_scale(divide_by), self._dev_index, raw),
                    "tftq_dequantize_scaled")
+
+
+def _post_scale(divide_by: float) -> float:
+    # torch divides a GPU tensor by a host scalar as a multiplication by the reciprocal,
+    # computed in double and rounded to fp32
+    divisor = float(divide_by)
+    return 1.0 / divisor if divisor != 0.0 else math.copysign(math.inf, divisor)
 
 
 def _check_packed(output: torch.Tensor, plan: _Plan, device: torch.device) -> None:
@@ -380,7 +542,20 @@ def fused_quantize_into_fp8(
     Returns:
         the packed uint8 tensor (``numel() % all_reduce_group_size == 0``)
     """
-    return prepare(inputs, all_reduce_group_size).quantize()
+    hit = _match_long_list(inputs, all_reduce_group_size, True)
+    if hit is None:
+        return prepare(inputs, all_reduce_group_size).quantize()
+    plan, device, ptrs = hit
+    out = torch.empty(plan.output_size, dtype=torch.uint8, device=device)
+    raw = _stream_of(device)
+    table, pointers, lock = _long_list_args(plan, device, raw, ptrs)
+    try:
+        rc = plan._lib.tftq_quantize(plan.handle, None, table, pointers, out.data_ptr(), plan.output_size,
+                                     device.index, raw)
+    finally:
+        lock.release()
+    _check(rc, "tftq_quantize")
+    return out
 
 
 def fused_dequantize_from_fp8(
@@ -397,7 +572,24 @@ def fused_dequantize_from_fp8(
     up with the bytes that dequantizing and then dividing each of them by that
     Python number on the GPU gives.
     """
-    prepare(inputs, all_reduce_group_size).dequantize(output, divide_by)
+    hit = _match_long_list(inputs, all_reduce_group_size, True)
+    if hit is None:
+        prepare(inputs, all_reduce_group_size).dequantize(output, divide_by)
+        return
+    plan, device, ptrs = hit
+    _check_packed(output, plan, device)
+    raw = _stream_of(device)
+    table, pointers, lock = _long_list_args(plan, device, raw, ptrs)
+    try:
+        if divide_by is None:
+            rc = plan._lib.tftq_dequantize(plan.handle, None, table, pointers, output.data_ptr(),
+                                           plan.output_size, device.index, raw)
+        else:
+            rc = plan._lib.tftq_dequantize_scaled(plan.handle, None, table, pointers, output.data_ptr(),
+                                                  plan.output_size, _post_scale(divide_by), device.index, raw)
+    finally:
+        lock.release()
+    _check(rc, "tftq_dequantize")
 
 
 def fused_reduce_fp8(
@@ -413,4 +605,14 @@ def fused_reduce_fp8(
     Any ``reduce_op`` other than SUM averages (quantization.py:682).
     ``inputs`` only supplies the shapes.
     """
-    prepare(inputs, all_reduce_group_size).reduce(output, all_reduce_rank, reduce_op)
+    hit = _match_long_list(inputs, all_reduce_group_size, False)
+    if hit is None:
+        prepare(inputs, all_reduce_group_size).reduce(output, all_reduce_rank, reduce_op)
+        return
+    plan, device, _ = hit
+    _check_packed(output, plan, device)
+    is_avg = 0 if reduce_op == ReduceOp.SUM else 1  # anything but SUM averages (:682)
+    raw = _stream_of(device)
+    table, _, _ = _long_list_args(plan, device, raw, None)
+    _check(plan._lib.tftq_reduce(plan.handle, table, output.data_ptr(), plan.output_size, int(all_reduce_rank),
+                                 is_avg, device.index, raw), "tftq_reduce")
