@@ -41,6 +41,11 @@ def test_scan_accepts_and_collects(pylist):
     ts[12] = torch.empty(0, 7)                          # empty
     ts[13] = torch.empty(40, 7)[3:7]                    # a view with a storage offset
     shapes, strides, ptrs = arrays(ts)
+    ts[14] = ts[14][:, 0]                               # 1-D: stands for its [k, 1] view ...
+    assert scan(pylist, ts, shapes, strides, ptrs) == 14
+    ts[14] = torch.empty(40)[::2]
+    ts[15] = torch.empty(9)
+    shapes, strides, ptrs = arrays([t if t.dim() == 2 else t.unsqueeze(1) for t in ts])  # ... of these sizes and strides
     assert scan(pylist, ts, shapes, strides, ptrs) == len(ts)
     assert list(ptrs) == [t.data_ptr() for t in ts]
     assert scan(pylist, ts, shapes, strides, None) == len(ts)   # no addresses wanted
@@ -55,7 +60,7 @@ def test_scan_stops_at_the_first_mismatch(pylist, what):
         "shape": lambda: torch.empty(4, 7),
         "stride": lambda: torch.empty(6, 4).t(),
         "dtype": lambda: torch.empty(4, 6, dtype=torch.float16),
-        "dim": lambda: torch.empty(24),
+        "dim": lambda: torch.empty(4, 6, 1),
         "none": lambda: None,
         "int": lambda: 5,
         "device": lambda: torch.empty(4, 6, device="meta"),

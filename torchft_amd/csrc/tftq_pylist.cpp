@@ -31,7 +31,7 @@ namespace {
 //   pointers  address of uint64[n] that receives the tensors' addresses (0: not wanted)
 //   n         length the list must have
 // Returns n when every element is a plain 2-D tensor of that dtype on that device with
-// those sizes and strides; the index of the first element that is not, otherwise (the
+// those sizes and strides (or the 1-D tensor that unsqueeze(1) turns into such a one); the index of the first element that is not, otherwise (the
 // addresses before it have then been written); -1 when `tensors` is not a list of n elements.
 PyObject *scan(PyObject *, PyObject *args)
 {
@@ -57,12 +57,14 @@ PyObject *scan(PyObject *, PyObject *args)
             // tensor subclasses that intercept operations (fake, functional, distributed
             // tensors) answer for themselves in Python
             if (!t.defined() || t.unsafeGetTensorImpl()->is_python_dispatch()) break;
-            if (t.dim() != 2 || t.scalar_type() != want) break;
+            const int64_t dim = t.dim();
+            if ((dim != 2 && dim != 1) || t.scalar_type() != want) break;
             const c10::Device d = t.device();
             if (device >= 0 ? (!d.is_cuda() || d.index() != device) : !d.is_cpu()) break;
             const c10::IntArrayRef sz = t.sizes(), st = t.strides();
-            if (sz[0] != shapes[2 * i] || sz[1] != shapes[2 * i + 1]) break;
-            if (st[0] != strides[2 * i] || st[1] != strides[2 * i + 1]) break;
+            // a 1-D tensor of k elements stands for its [k, 1] view (quantization.py:487-488)
+            if (sz[0] != shapes[2 * i] || (dim == 2 ? sz[1] : 1) != shapes[2 * i + 1]) break;
+            if (st[0] != strides[2 * i] || (dim == 2 ? st[1] : 1) != strides[2 * i + 1]) break;
             if (pointers) pointers[i] = static_cast<uint64_t>(reinterpret_cast<uintptr_t>(t.data_ptr()));
         }
     } catch (...) {
