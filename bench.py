@@ -46,12 +46,14 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--sets", type=int, default=3, help="buffer sets the steps rotate over")
     ap.add_argument("--rank", type=int, default=None)
-    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat", "shape", "ceiling"],
+    ap.add_argument("--config", default="3", choices=["2", "3", "4", "5", "flat", "shape", "ceiling", "ceiling4"],
                     help="workload: 3 = Llama-3-8B layer bucket (the headline, default); 2, 4, 5 = the "
                          "other GPU configurations; flat = one 1-D fp32 tensor of 64 Mi elements "
                          "(what a bucketised DiLoCo all-reduce passes); shape = --shape; ceiling = "
                          "streaming kernels without arithmetic for the read : write mixes of the "
-                         "stages, at the headline workload's footprint, beside the product kernels")
+                         "stages, at the headline workload's footprint, beside the product kernels; "
+                         "ceiling4 = the accesses of reduce on configuration 4 (4 peers, rows of 2052 and "
+                         "5636 bytes) without arithmetic, beside the product's reduce on that configuration")
     ap.add_argument("--shape", default="53248x4096",
                     help="with --config shape: ROWSxCOLS[,ROWSxCOLS...], N(0, 0.02) values")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16", "float32"],
@@ -173,10 +175,10 @@ def run_ceilings(args) -> int:
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
 
     def timed(launch, nbytes):
-        for i in range(args.warmup):
-            launch(i)
         pairs = [(ev(), ev()) for _ in range(args.steps)]
         torch.cuda.synchronize()
+        for i in range(args.warmup):  # the timed launches are queued behind these: no idle GPU in between
+            launch(i)
         for i, (a, b) in enumerate(pairs):
             a.record(stream)
             launch(i)
@@ -207,9 +209,9 @@ def run_ceilings(args) -> int:
              ("1:4 read:write, 4 steps per lane", 14, 26624, 0, BOTH, NT),
              ("8:1 read:write, one contiguous source (reduce, 8 peers)", 6, 6656, 0, BOTH, BOTH),
              ("reduce's accesses: 8 slots, 4100-byte rows, in place, an eighth of the rows per XCD",
-              7, rows, 1, NT, PLAIN),
-             ("reduce's accesses, rows in workgroup order", 7, rows, 0, NT, PLAIN),
-             ("reduce's accesses, an eighth per XCD, wavefronts start on 128-byte lines", 8, rows, 1, NT, PLAIN),
+              7, rows, 1, NT, BOTH),
+             ("reduce's accesses, rows in workgroup order", 7, rows, 0, NT, BOTH),
+             ("reduce's accesses, an eighth per XCD, wavefronts start on 128-byte lines", 8, rows, 1, NT, BOTH),
              ("quantize's accesses: 8 KB rows -> 4100-byte packed rows through LDS, rows in workgroup order",
               10, 8 * rows, 0, NT, NT),
              ("quantize's accesses, packed rows straight from the registers (plain stores)",
@@ -232,6 +234,8 @@ def run_ceilings(args) -> int:
                 if kind < 7 or kind >= 11:
                     label += (", streaming loads" if ntl else ", plain loads") if rb.value else ""
                     label += (", streaming stores" if nts else ", plain stores") if wb.value else ""
+                elif kind in (7, 8):
+                    label += ", streaming stores" if nts else ", plain stores"
                 r = timed(launch, rb.value + wb.value)
                 r["read_bytes"], r["write_bytes"], r["kind"] = rb.value, wb.value, kind
                 ceilings[label] = r
@@ -273,6 +277,84 @@ def run_ceilings(args) -> int:
                                   f"packed, 8 slots); {nsets} rotating buffer sets"},
            "ceilings": ceilings, "product": product}
     print(json.dumps(out))
+    return 0
+
+
+def run_ceiling4(args, sets, ws, rank, op, ab) -> int:
+    """The accesses of reduce on configuration 4 and nothing else (k_reduce_pattern_mix of
+    torchft_amd/csrc/tftq_ceiling.hip: 4 slots, 103 296 rows of 2052 bytes handled by a wavefront
+    each and 11 264 rows of 5636 bytes handled by a workgroup each, in place, work handed to the
+    XCDs in chunks of 64 workgroups), a plain 4 : 1 copy of the same bytes, and the product's
+    reduce on configuration 4: every kernel alone in a loop that rotates over the buffer sets,
+    HIP events around each launch."""
+    import ctypes
+
+    import torch
+
+    from torchft_amd import _build, quantization as q
+
+    if not os.path.exists(_build.CEILING_LIB_PATH):
+        _build.build_library()
+    C = ctypes.CDLL(_build.CEILING_LIB_PATH)
+    C.tftq_ceiling_reduce_mix.argtypes = [ctypes.c_void_p, ctypes.c_int64] + [ctypes.c_int] * 4 + [
+        ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p]
+    C.tftq_ceiling_launch.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                      ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    stream = torch.cuda.current_stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
+
+    def timed(launch, nbytes):
+        pairs = [(ev(), ev()) for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        for i in range(args.warmup):  # the timed launches are queued behind these: no idle GPU in between
+            launch(i)
+        for i, (a, b) in enumerate(pairs):
+            a.record(stream)
+            launch(i)
+            b.record(stream)
+        torch.cuda.synchronize()
+        us = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
+        mean = sum(us) / len(us)
+        return {"us": round(mean, 2), "us_min": round(us[0], 2), "us_median": round(us[len(us) // 2], 2), "bytes": nbytes,
+                "GBs": round(nbytes / mean / 1e3, 1), "frac_of_peak": round(nbytes / mean / 1e3 / HBM_PEAK_GBS, 4)}
+
+    out = {}
+    # the pattern kernels overwrite the own slot with bytes that are no scales and codes: they
+    # run on copies of the received buffers
+    scratch = [s_["recv"].clone() for s_ in sets]
+    rows_a, rb_a, rows_b, rb_b = 103296, 2052, 11264, 5636  # rows per slot of the two row lengths
+    slot = sets[0]["recv"].numel() // ws
+    assert rows_a * rb_a + rows_b * rb_b <= slot
+    nbytes = (ws + 1) * (rows_a * rb_a + rows_b * rb_b)
+    for nts in (0, 1):
+        def launch(i, nts=nts):
+            rc = C.tftq_ceiling_reduce_mix(scratch[i % len(sets)].data_ptr(), slot, ws, rank, rows_a, rb_a,
+                                           rows_b * rb_b, rows_b, rb_b, 0, 6, 1, nts, sp)
+            assert rc == 0, rc
+        out["reduce's accesses, " + ("streaming" if nts else "plain") + " stores"] = timed(launch, nbytes)
+    # a plain 4 : 1 copy of about the same bytes: 33 623 chunks of 32 KB read, 8 KB written
+    units = nbytes // (5 * 8192)
+    for nts in (0, 1):
+        def launch(i, nts=nts):
+            a, b = scratch[i % len(sets)], sets[i % len(sets)]["gathered"]
+            rc = C.tftq_ceiling_launch(4, a.data_ptr(), b.data_ptr(), units, 0, 0, 0, 0, 1, nts, sp)
+            assert rc == 0, rc
+        out["4:1 copy, streaming loads, " + ("streaming" if nts else "plain") + " stores"] = timed(launch, units * 5 * 8192)
+    del scratch
+    # (last: by now the threads of the CPU checker that the parity gate ran have gone to sleep, and
+    # the host queues its launches ahead of the GPU)
+    out["product reduce"] = timed(lambda i: q.fused_reduce_fp8(sets[i % len(sets)]["tensors"], sets[i % len(sets)]["recv"],
+                                                              ws, rank, op), ab["reduce"])
+    best = max(v["GBs"] for k, v in out.items() if k.startswith("reduce's accesses"))
+    out["product reduce"]["of_own_accesses"] = round(out["product reduce"]["GBs"] / best, 4)
+    print(json.dumps({"metric": "reduce on configuration 4: the product kernel and kernels that only make its accesses, "
+                                "each alone, HBM GB/s on 1 MI355X", "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup,
+                      "config": {"workload": f"configuration 4 (ws=4, slot of {slot} bytes); {len(sets)} rotating buffer sets"},
+                      "kernels": out}))
     return 0
 
 
@@ -332,9 +414,10 @@ def main() -> int:
 
         table["shape"] = (make_shape, args.ws, ReduceOp.AVG,
                           f"tensors {args.shape} {args.dtype}, N(0, 0.02), ws={args.ws}, AVG")
+    table["ceiling4"] = table["4"]
     make, ws, op, workload_name = table[args.config]
     rank = args.rank if args.rank is not None else min(3, ws - 1)
-    if args.config == "4":
+    if args.config in ("4", "ceiling4"):
         args.sets = min(args.sets, 2)
 
     # ---- buffer sets: tensors, received buffer B, gathered buffer G ----------
@@ -380,6 +463,9 @@ def main() -> int:
     if not ok:
         print("bench.py: GPU results differ from the CPU checker", file=sys.stderr)
         return 1
+
+    if args.config == "ceiling4":
+        return run_ceiling4(args, sets, ws, rank, op, ab)
 
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
     STAGES = ("quantize", "reduce", "dequantize")

@@ -23,6 +23,8 @@
 //   RED      reduce on rows of up to 4096 codes: one workgroup per row, a lane loads one
 //            16-byte vector of each of 8 sources one slot apart (rows of row_bytes, payload
 //            4 bytes behind the row start), the result goes over source `rank` in place
+//   (k_reduce_pattern_mix, tftq_ceiling_reduce_mix: the same for a group of 4 and a slot of
+//            two row lengths, the shape of the reduce of an fp32 pseudo-gradient)
 //   RED_LINE RED with the 1 KB that a wavefront accesses moved down to a 128-byte line:
 //            what it costs that packed rows start anywhere
 //   DEQ      dequantize on 16-bit rows of 4096 columns: one wavefront per row, a lane loads
@@ -129,7 +131,7 @@ __device__ __forceinline__ int piece_of(int per_xcd)
     return per_xcd > 0 ? (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
 }
 
-template <bool NTL, bool LINE>
+template <bool NTL, bool LINE, bool NTS>
 __global__ __launch_bounds__(256) void k_reduce_pattern(uint8_t *buf, int64_t slot_size, int rows, int row_bytes,
                                                         int rank, int per_xcd)
 {
@@ -155,8 +157,71 @@ __global__ __launch_bounds__(256) void k_reduce_pattern(uint8_t *buf, int64_t sl
     GLOBAL u32 *orow = (GLOBAL u32 *)(uint64_t)(buf + rank * slot_size + off);
     uint64_t oaddr = (uint64_t)(orow + 1 + doff);
     if (LINE) oaddr = ((uint64_t)(orow + 1 + (doff & ~255)) & ~(uint64_t)127) + 16 * (t & 63);
-    if (4 * t < ndw) *(GLOBAL u32x4_a4 *)oaddr = a;
+    if (4 * t < ndw) {
+        if (NTS) __builtin_nontemporal_store(a, (GLOBAL u32x4_a4 *)oaddr);
+        else *(GLOBAL u32x4_a4 *)oaddr = a;
+    }
     if (t == 0) orow[0] = a.x;
+}
+
+// Reduce's accesses on a slot that holds two kinds of rows, for a group of WS peers (WS * UNITS
+// = 8 loads per lane): rows_b rows of row_bytes_b (more than 1024 and at most 2048 payload
+// dwords: one workgroup per row, two vectors per lane and peer in the lower wavefronts, as many
+// as the row needs in the upper ones) from byte off_b of every slot, handed out first, then
+// rows_a rows of row_bytes_a (at most 512 payload dwords: one wavefront per row, two vectors per
+// lane and peer) from byte off_a.  Chunks of 2^chunk_shift consecutive workgroups go to the 8
+// XCDs in turn, as the product hands out the work of long tensor lists.
+template <int WS, bool NTL, bool NTS>
+__global__ __launch_bounds__(256) void k_reduce_pattern_mix(uint8_t *buf, int64_t slot_size, int rank, int rows_a,
+                                                            int row_bytes_a, int64_t off_a, int rows_b, int row_bytes_b,
+                                                            int64_t off_b, int chunk_shift, int nwg)
+{
+    constexpr int UNITS = 8 / WS;
+    const int i = (int)(blockIdx.x >> 3), x = (int)(blockIdx.x & 7), cs = chunk_shift;
+    const int vb = ((((i >> cs) << 3) + x) << cs) + (i & ((1 << cs) - 1));
+    if (vb >= nwg) return;
+    const int t = threadIdx.x, wave = t >> 6;
+    int team, lane, ndw, units = UNITS;
+    int64_t off;
+    if (vb < rows_b) {
+        team = 256; lane = t;
+        ndw = (row_bytes_b >> 2) - 1;
+        off = off_b + (int64_t)vb * row_bytes_b;
+        units = min(UNITS, max(1, (ndw - 256 * wave + 1023) >> 10));
+    } else {
+        const int j = (vb - rows_b) * 4 + wave;
+        if (j >= rows_a) return;
+        team = 64; lane = t & 63;
+        ndw = (row_bytes_a >> 2) - 1;
+        off = off_a + (int64_t)j * row_bytes_a;
+    }
+    int doff[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) doff[u] = min(4 * (u * team + lane), ndw - 4);
+    u32x4 w[WS][UNITS];
+#pragma unroll
+    for (int k = 0; k < WS; k++) {
+        int peer = rank + k;
+        if (peer >= WS) peer -= WS;
+        GLOBAL const u32 *pv = (GLOBAL const u32 *)(uint64_t)(buf + peer * slot_size + off) + 1;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            GLOBAL const u32x4_a4 *q = (GLOBAL const u32x4_a4 *)(pv + doff[u < units ? u : 0]);
+            w[k][u] = NTL ? __builtin_nontemporal_load(q) : *q;
+        }
+    }
+    GLOBAL u32 *orow = (GLOBAL u32 *)(uint64_t)(buf + rank * slot_size + off);
+#pragma unroll
+    for (int u = 0; u < UNITS; u++) {
+        u32x4 a = w[0][u];
+#pragma unroll
+        for (int k = 1; k < WS; k++) a ^= w[k][u];
+        if (u < units && 4 * (u * team + lane) < ndw) {
+            if (NTS) __builtin_nontemporal_store(a, (GLOBAL u32x4_a4 *)(orow + 1 + doff[u]));
+            else *(GLOBAL u32x4_a4 *)(orow + 1 + doff[u]) = a;
+        }
+        if (u == 0 && lane == 0) orow[0] = a.x;
+    }
 }
 
 template <bool NTL, bool NTS>
@@ -258,7 +323,7 @@ extern "C" int tftq_ceiling_bytes(int kind, int64_t units, int row_bytes, int64_
 // a multiple of 128), src is not used, 20 <= row_bytes <= 4100.  DEQ: src holds the packed rows
 // (row_bytes >= 4100 apart), dst the rows of 8192 bytes.  QNT: src holds rows of 8192 bytes, dst
 // the packed rows (row_bytes = 4100, units a multiple of 4).  nt_loads / nt_stores pick streaming
-// (nontemporal) accesses; the patterns store as the product does (RED plain, DEQ per nt_stores).
+// (nontemporal) accesses (RED, RED_LINE: of the codes; the scale dword is a plain store).
 // Returns 0, a hipError_t, or -1 for bad arguments.
 extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t units, int64_t slot_size,
                                    int row_bytes, int rank, int eighths, int nt_loads, int nt_stores, void *stream)
@@ -297,13 +362,16 @@ extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t
         const int px = eighths ? (int)((units + 7) / 8) : 0;
         const dim3 g(eighths ? (unsigned)(8 * px) : (unsigned)units);
         const int rows = (int)units;
-        if (kind == C_RED) {
-            if (nt_loads) hipLaunchKernelGGL((k_reduce_pattern<true, false>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);
-            else hipLaunchKernelGGL((k_reduce_pattern<false, false>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);
-        } else {
-            if (nt_loads) hipLaunchKernelGGL((k_reduce_pattern<true, true>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);
-            else hipLaunchKernelGGL((k_reduce_pattern<false, true>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);
-        }
+#define TFTQ_RED(LINE)                                                                                              \
+    do {                                                                                                            \
+        if (nt_loads && nt_stores) hipLaunchKernelGGL((k_reduce_pattern<true, LINE, true>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);        \
+        else if (nt_loads) hipLaunchKernelGGL((k_reduce_pattern<true, LINE, false>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);              \
+        else if (nt_stores) hipLaunchKernelGGL((k_reduce_pattern<false, LINE, true>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);             \
+        else hipLaunchKernelGGL((k_reduce_pattern<false, LINE, false>), g, block, 0, s, b, slot_size, rows, row_bytes, rank, px);                           \
+    } while (0)
+        if (kind == C_RED) TFTQ_RED(false);
+        else TFTQ_RED(true);
+#undef TFTQ_RED
         break;
     }
     case C_DEQ: {
@@ -333,5 +401,42 @@ extern "C" int tftq_ceiling_launch(int kind, const void *src, void *dst, int64_t
     default: return -1;
     }
 #undef TFTQ_C
+    return (int)hipGetLastError();
+}
+
+// One launch of k_reduce_pattern_mix on `stream` (see there): buf holds ws slots of slot_size
+// bytes and is updated in place; ws is 4 or 8; nt_loads / nt_stores pick streaming accesses for
+// the codes (the scale dword is always a plain store).  Reads ws times, writes once, the
+// rows_a * row_bytes_a + rows_b * row_bytes_b bytes of a slot's rows.
+extern "C" int tftq_ceiling_reduce_mix(void *buf, int64_t slot_size, int ws, int rank, int rows_a, int row_bytes_a,
+                                       int64_t off_a, int rows_b, int row_bytes_b, int64_t off_b, int chunk_shift,
+                                       int nt_loads, int nt_stores, void *stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    if (!buf || (ws != 4 && ws != 8) || rank < 0 || rank >= ws || rows_a < 0 || rows_b < 0) return -1;
+    if ((row_bytes_a & 3) || (row_bytes_b & 3) || row_bytes_a < 20 || row_bytes_a > 2052) return -1;
+    if (rows_b > 0 && (row_bytes_b <= 4100 || row_bytes_b > 8196)) return -1;
+    if (chunk_shift < 0 || chunk_shift > 16) return -1;
+    const int nwg = rows_b + (rows_a + 3) / 4;
+    if (nwg == 0) return 0;
+    const int chunk = 1 << chunk_shift;
+    const int chunks = (nwg + chunk - 1) / chunk;
+    const int per_xcd = (chunks + 7) / 8 * chunk;
+    const dim3 grid((unsigned)(8 * per_xcd)), block(256);
+    uint8_t *b = (uint8_t *)buf;
+#define TFTQ_MIX(WS, NTL, NTS)                                                                                        \
+    hipLaunchKernelGGL((k_reduce_pattern_mix<WS, NTL, NTS>), grid, block, 0, s, b, slot_size, rank, rows_a, row_bytes_a, \
+                       off_a, rows_b, row_bytes_b, off_b, chunk_shift, nwg)
+#define TFTQ_MIX_W(WS)                                                                     \
+    do {                                                                                   \
+        if (nt_loads && nt_stores) TFTQ_MIX(WS, true, true);                               \
+        else if (nt_loads) TFTQ_MIX(WS, true, false);                                      \
+        else if (nt_stores) TFTQ_MIX(WS, false, true);                                     \
+        else TFTQ_MIX(WS, false, false);                                                   \
+    } while (0)
+    if (ws == 4) TFTQ_MIX_W(4);
+    else TFTQ_MIX_W(8);
+#undef TFTQ_MIX_W
+#undef TFTQ_MIX
     return (int)hipGetLastError();
 }
