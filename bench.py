@@ -59,11 +59,15 @@ def parse_args():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float16", "float32"],
                     help="with --config shape")
     ap.add_argument("--ws", type=int, default=8, help="with --config shape: group size (reduce AVG)")
-    ap.add_argument("--api", default="named", choices=["named", "prepared"],
+    ap.add_argument("--api", default="named", choices=["named", "prepared", "collective"],
                     help="named: the three functions the reference names, as torchft/collectives.py calls "
                          "them (default); prepared: torchft_amd.quantization.prepare() once per tensor "
                          "list, then the bucket's quantize (into a buffer kept from step to step) / "
-                         "reduce / dequantize: the form for a bucket that is reduced every step")
+                         "reduce / dequantize: the form for a bucket that is reduced every step; "
+                         "collective: torchft_amd.collectives.allreduce_quantized on the workload (configs 2, 3, "
+                         "shape), through torch.distributed's RCCL process group with this process as its only "
+                         "rank and through a group of 8 ranks simulated by threads on the one GPU: wall time "
+                         "per call against the time of its kernels, and where the host's time goes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a counter "
@@ -280,6 +284,268 @@ def run_ceilings(args) -> int:
     return 0
 
 
+class _TimedGroup:
+    """A process group seen through a stopwatch: host time of every collective call and of
+    every wait() on the work objects they return (torchft_amd.collectives calls wait() twice
+    per all-reduce), and device events around each collective."""
+
+    def __init__(self, pg, log):
+        self._pg, self._log = pg, log
+
+    def rank(self):
+        return self._pg.rank()
+
+    def size(self):
+        return self._pg.size()
+
+    def _call(self, name, fn, *a):
+        import torch
+        log = self._log
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        stream = torch.cuda.current_stream()
+        e0.record(stream)
+        t0 = time.perf_counter()
+        work = fn(*a)
+        log[name + " call"] = time.perf_counter() - t0
+        outer = self
+
+        class Work:
+            def wait(self, *wa):
+                t = time.perf_counter()
+                r = work.wait(*wa)
+                log[name + " wait()"] = log.get(name + " wait()", 0.0) + time.perf_counter() - t
+                e1.record(torch.cuda.current_stream())
+                outer._log.setdefault("events", {})[name] = (e0, e1)
+                return r
+
+            def get_future(self):
+                fut = work.get_future()
+                t_asked = time.perf_counter()
+                fut.add_done_callback(lambda f: log.__setitem__(name + " future done after", time.perf_counter() - t_asked))
+                return fut
+
+        return Work()
+
+    def alltoall_base(self, *a):
+        return self._call("all-to-all", self._pg.alltoall_base, *a)
+
+    def allgather_into_tensor_coalesced(self, *a):
+        return self._call("all-gather", self._pg.allgather_into_tensor_coalesced, *a)
+
+
+class _TimedBucket:
+    """A prepared bucket seen through a stopwatch: host time and device events of the three launches."""
+
+    def __init__(self, bucket, log):
+        self._b, self._log = bucket, log
+        self.ws = bucket.ws
+
+    def matches(self, tensors):
+        t = time.perf_counter()
+        ok = self._b.matches(tensors)
+        self._log["bucket.matches()"] = time.perf_counter() - t
+        return ok
+
+    def _launch(self, name, fn, *a):
+        import torch
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        stream = torch.cuda.current_stream()
+        e0.record(stream)
+        t = time.perf_counter()
+        r = fn(*a)
+        self._log[name + " launch"] = time.perf_counter() - t
+        self._log[name + " at"] = t
+        e1.record(stream)
+        self._log.setdefault("events", {})[name] = (e0, e1)
+        return r
+
+    def quantize(self, *a):
+        return self._launch("quantize", self._b.quantize, *a)
+
+    def reduce(self, *a):
+        return self._launch("reduce", self._b.reduce, *a)
+
+    def dequantize(self, *a):
+        return self._launch("dequantize", self._b.dequantize, *a)
+
+
+def run_collective(args, make, op, workload_name) -> int:
+    """allreduce_quantized (torchft/collectives.py:297-415) end to end on one GPU."""
+    import socket
+    import threading
+
+    import torch
+    import torch.distributed as dist
+    from torch.distributed import ReduceOp
+
+    import sim_pg
+    import workloads
+    from torchft_amd import collectives as col, quantization as q
+
+    dev = "cuda"
+    nsets = max(2, args.sets)
+    K, W = args.steps, args.warmup
+
+    def measure(pg_of, ws, rank_threads):
+        """Per rank: W + K calls one after the other, each waited for to the end (latency),
+        then K calls queued back to back (throughput).  Returns rank 0's figures."""
+        result = {}
+
+        def rank_fn(r):
+            torch.cuda.set_device(0)
+            pg = pg_of(r)
+            stream = torch.cuda.Stream()
+            sets = [make(1000 * k + r) for k in range(nsets)]
+            buckets = [q.prepare(t, ws) for t in sets]
+            ab = workloads.algorithmic_bytes(sets[0], ws)
+            logs = []
+
+            def one_call(i, timed):
+                log = {}
+                tensors = sets[i % nsets]
+                group = _TimedGroup(pg, log) if timed else pg
+                bucket = _TimedBucket(buckets[i % nsets], log) if timed else buckets[i % nsets]
+                t0 = time.perf_counter()
+                work = col.allreduce_quantized(tensors, op, group, stream, prepared=bucket)
+                log["returned after"] = time.perf_counter() - t0
+                work.wait()
+                work.get_future().wait()
+                stream.synchronize()
+                log["wall"] = time.perf_counter() - t0
+                log["t0"] = t0
+                return log
+
+            for i in range(W):
+                one_call(i, False)
+            torch.cuda.synchronize()
+            plain = [one_call(i, False)["wall"] for i in range(K)]     # no stopwatch in the way
+            logs = [one_call(i, True) for i in range(K)]
+            # back to back: K calls queued, then everything waited for
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            works = [col.allreduce_quantized(sets[i % nsets], op, pg, stream, prepared=buckets[i % nsets])
+                     for i in range(K)]
+            queued = time.perf_counter() - t0
+            for w in works:
+                w.wait()
+                w.get_future().wait()
+            stream.synchronize()
+            back_to_back = (time.perf_counter() - t0) / K
+            if r != 0:
+                return
+            us = lambda x: round(x * 1e6, 1)  # noqa: E731
+            mean = lambda xs: sum(xs) / len(xs)  # noqa: E731
+            host = {}
+            for key in ("bucket.matches()", "quantize launch", "all-to-all call", "all-to-all wait()", "reduce launch",
+                        "all-gather call", "all-gather wait()", "returned after", "all-gather future done after",
+                        "dequantize launch"):
+                vals = [l[key] for l in logs if key in l]
+                if vals:
+                    host[key + " us"] = us(mean(vals))
+            host["dequantize queued after the call started us"] = us(mean([l["dequantize at"] - l["t0"] for l in logs]))
+            gpu = {}
+            for name in ("quantize", "all-to-all", "reduce", "all-gather", "dequantize"):
+                vals = [l["events"][name][0].elapsed_time(l["events"][name][1]) * 1e-3 for l in logs if name in l.get("events", {})]
+                if vals:
+                    gpu[name + " us"] = us(mean(vals))
+            first_to_last = [l["events"]["quantize"][0].elapsed_time(l["events"]["dequantize"][1]) * 1e-3 for l in logs]
+            kernels = sum(gpu.get(k + " us", 0.0) for k in ("quantize", "reduce", "dequantize"))
+            exchange = sum(gpu.get(k + " us", 0.0) for k in ("all-to-all", "all-gather"))
+            # the receive buffer (collectives.py:367 allocates it on every call)
+            t = time.perf_counter()
+            for _ in range(200):
+                buf = torch.empty(buckets[0].output_size, dtype=torch.uint8, device=dev)
+            alloc = (time.perf_counter() - t) / 200
+            del buf
+            # the three kernels alone, queued back to back (no idle GPU between the events)
+            alone = {}
+            b0 = buckets[0]
+            packed0 = b0.quantize()
+            for name, fn in (("quantize", lambda: b0.quantize(out=packed0)),
+                             ("reduce", lambda: b0.reduce(packed0, pg.rank(), op)),
+                             ("dequantize", lambda: b0.dequantize(packed0))):
+                pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+                with torch.cuda.stream(stream):
+                    for _ in range(W):
+                        fn()
+                    for a, b in pairs:
+                        a.record(stream)
+                        fn()
+                        b.record(stream)
+                stream.synchronize()
+                alone[name + " us"] = us(mean([a.elapsed_time(b) * 1e-3 for a, b in pairs]))
+            result.update({
+                "ranks": ws,
+                "wall_us_per_call": us(mean(plain)),
+                "wall_us_per_call_with_stopwatch": us(mean([l["wall"] for l in logs])),
+                "back_to_back_us_per_call": us(back_to_back),
+                "host_us_to_queue_one_call_back_to_back": us(queued / K),
+                "kernels_alone_us": alone,
+                "kernels_alone_sum_us": round(sum(alone.values()), 1),
+                "gpu_us_first_kernel_to_last_with_stopwatch": us(mean(first_to_last)),
+                "gpu_us_between_events_with_stopwatch": gpu,
+                "host_us_with_stopwatch": host,
+                "receive_buffer_allocation_us": us(alloc),
+                "algorithmic_bytes": sum(ab.values()),
+                "note": "wall_us_per_call: call, work.wait(), future.wait(), stream.synchronize(), one call after the "
+                        "other; back_to_back: K calls queued, then all waited for; the stopwatch pass wraps the group "
+                        "and the bucket (host timers, device events) and is slower for it; device events around a "
+                        "launch on an idle GPU include the launch latency",
+            })
+
+        if rank_threads == 1:
+            rank_fn(0)
+        else:
+            errors = []
+
+            def body(r):
+                try:
+                    rank_fn(r)
+                except BaseException as e:  # noqa: BLE001
+                    errors.append(e)
+                    group.barrier.abort()
+
+            threads = [threading.Thread(target=body, args=(r,)) for r in range(rank_threads)]
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join()
+            if errors:
+                raise errors[0]
+        return result
+
+    out = {}
+    if dist.is_nccl_available():
+        with socket.socket() as sock:
+            sock.bind(("127.0.0.1", 0))
+            port = sock.getsockname()[1]
+        # RCCL prints a banner on standard output when it creates its communicator: this command's
+        # standard output is one line of JSON, so the descriptor points at standard error meanwhile
+        sys.stdout.flush()
+        saved = os.dup(1)
+        os.dup2(2, 1)
+        try:
+            dist.init_process_group("nccl", init_method=f"tcp://127.0.0.1:{port}", rank=0, world_size=1,
+                                    device_id=torch.device("cuda:0"))
+            try:
+                pg = dist.distributed_c10d._get_default_group()
+                out["RCCL process group, this process its only rank"] = measure(lambda r: pg, 1, 1)
+            finally:
+                dist.destroy_process_group()
+        finally:
+            sys.stdout.flush()
+            os.dup2(saved, 1)
+            os.close(saved)
+    group = sim_pg.SimGroup(8)
+    out["8 ranks simulated by threads on the one GPU (rank 0's figures; the GPU serves all 8)"] = \
+        measure(group.rank, 8, 8)
+    print(json.dumps({"metric": "allreduce_quantized end to end on 1 MI355X: wall time per call against its kernels",
+                      "unit": "us", "n_gpus": 1, "steps": K, "warmup": W,
+                      "config": {"workload": workload_name, "api": "collective", "buffer_sets": nsets},
+                      "groups": out}))
+    return 0
+
+
 def run_ceiling4(args, sets, ws, rank, op, ab) -> int:
     """The accesses of reduce on configuration 4 and nothing else (k_reduce_pattern_mix of
     torchft_amd/csrc/tftq_ceiling.hip: 4 slots, 103 296 rows of 2052 bytes handled by a wavefront
@@ -416,6 +682,11 @@ def main() -> int:
                           f"tensors {args.shape} {args.dtype}, N(0, 0.02), ws={args.ws}, AVG")
     table["ceiling4"] = table["4"]
     make, ws, op, workload_name = table[args.config]
+    if args.api == "collective":
+        if args.config not in ("2", "3", "shape"):
+            print("bench.py --api collective runs configurations 2, 3 and shape", file=sys.stderr)
+            return 2
+        return run_collective(args, make, op, workload_name)
     rank = args.rank if args.rank is not None else min(3, ws - 1)
     if args.config in ("4", "ceiling4"):
         args.sets = min(args.sets, 2)

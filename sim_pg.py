@@ -1,4 +1,4 @@
-"""A process group simulated inside one process, for testing the host
+"""A process group simulated inside one process, for testing and timing the host
 orchestration of the quantized collectives on a single GPU.
 
 Every rank is a thread (as in the reference's own collective tests,

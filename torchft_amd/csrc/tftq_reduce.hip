@@ -616,17 +616,25 @@ DEV void reduce_rows_roll(const Seg &s, const KParams &p, int j, int lane, float
 #pragma unroll
         for (int u = 0; u < UNITS; u++) w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + boff[u]));
     }
-    float acc[UNITS][16];
-#pragma unroll
-    for (int u = 0; u < UNITS; u++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
+    float acc[UNITS][16];  // set by the first peer
     const float sc = raw_scale == 0.0f ? 1.0f : raw_scale;  // padding rows (:419)
     const DivCoef c = make_div(sc);
     const bool row_fast = __builtin_amdgcn_ballot_w64(!c.fast) == 0;  // same in all wavefronts of the team
     if (row_fast) {
+        {   // the first peer (a group of one reads it a second time and ignores that)
+            const float pr = team_bcast<TEAM>(c.r, 0), pl = team_bcast<TEAM>(c.r_lo, 0);
+            GLOBAL const uint8_t *pv = (GLOBAL const uint8_t *)(peer_row(p, min(1, ws - 1), off) + 1);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) {
+                u32x4 x = w[u];
+                asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
+                w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + boff[u]));
+                x.w &= padmask[u];
+                accumulate16<true>(acc[u], x, pr, pl);
+            }
+        }
 #pragma nounroll
-        for (int k = 0; k + 1 < ws; k++) {
+        for (int k = 1; k + 1 < ws; k++) {
             const float pr = team_bcast<TEAM>(c.r, k), pl = team_bcast<TEAM>(c.r_lo, k);
             GLOBAL const uint8_t *pv = (GLOBAL const uint8_t *)(peer_row(p, k + 1, off) + 1);
 #pragma unroll
@@ -638,7 +646,7 @@ DEV void reduce_rows_roll(const Seg &s, const KParams &p, int j, int lane, float
                 accumulate16(acc[u], x, pr, pl);
             }
         }
-        {
+        if (ws > 1) {
             const float pr = team_bcast<TEAM>(c.r, ws - 1), pl = team_bcast<TEAM>(c.r_lo, ws - 1);
 #pragma unroll
             for (int u = 0; u < UNITS; u++) {
@@ -717,7 +725,7 @@ DEV void reduce_rows_at_once(const Seg &s, const KParams &p, int j0, int lane, f
 #pragma unroll
         for (int u = 0; u < UNITS; u++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[r][u][e] = 0.0f;
+            for (int e = 0; e < 16; e++) acc[r][u][e] = 0.0f;  // a slow row's sums are not used
         amax[r] = 0.0f;
         if (fast[r]) {
 #pragma unroll
@@ -728,7 +736,8 @@ DEV void reduce_rows_at_once(const Seg &s, const KParams &p, int j0, int lane, f
                     for (int u = 0; u < UNITS; u++) {
                         u32x4 v = w[r][k][u];
                         v.w &= padmask[u];
-                        accumulate16(acc[r][u], v, pr, pl);
+                        if (k == 0) accumulate16<true>(acc[r][u], v, pr, pl);  // the first peer sets the sums
+                        else accumulate16(acc[r][u], v, pr, pl);
                     }
                 }
             }
