@@ -66,6 +66,7 @@ extern "C" {
 #define TFTQ_E_NOTABLE (-6)  /* a list longer than TFTQ_N_INLINE needs `table` (and `pointers`) */
 #define TFTQ_E_ARCH (-7)     /* the device is not gfx950 */
 #define TFTQ_E_TOOBIG (-8)   /* tftq_reduce_static: the list's table exceeds TFTQ_STATIC_TABLE_BYTES */
+#define TFTQ_E_BUSY (-9)     /* tftq_reduce_static: a call on another stream of the device has not finished */
 
 typedef struct tftq_plan tftq_plan;
 
@@ -123,7 +124,9 @@ int tftq_plan_n_tensors(const tftq_plan *plan);
  *             here with small kernels on `stream` (the host array is read
  *             before the call returns; nothing blocks); with tensors == NULL it
  *             uses what `pointers` already holds.  One `pointers` buffer must
- *             not be written by calls that overlap in time.
+ *             not be written by calls that overlap in time.  All arguments are
+ *             checked before the addresses are written; a call whose kernel launch
+ *             then fails with a hipError_t has still rewritten `pointers`.
  * For short lists both are ignored (pass NULL) and tftq_plan_table_bytes() is 0.
  */
 int64_t tftq_plan_table_bytes(const tftq_plan *plan);
@@ -190,9 +193,13 @@ int tftq_dequantize_scaled(const tftq_plan *plan, void *const *tensors, const vo
  * costs one small kernel per 3584 bytes of table in front of the reduce kernel.  The
  * array's address on a device is looked up once, by tftq_check_device() for that device
  * or else by the first call there (which should then not run under stream capture).
- * All calls on one device share that array: calls that overlap in time on one device
- * (different streams or threads) race on it and must be serialised by the caller.
- * Results are those of tftq_reduce.
+ * All calls on one device share that array.  Calls on one stream are ordered by the stream.
+ * A call on another stream than the last one, while the last one's kernel has not finished,
+ * queues nothing and returns TFTQ_E_BUSY (wait for that stream, or make this one wait for it,
+ * and call again); calls from several threads are taken one at a time.  Calls that a stream
+ * capture records are not checked against each other or against later calls: replays of
+ * graphs that hold such calls, and eager calls beside them, must be serialised by the
+ * caller.  Results are those of tftq_reduce.
  */
 #define TFTQ_STATIC_TABLE_BYTES (512 * 1024)
 int tftq_reduce_static(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank,

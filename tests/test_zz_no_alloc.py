@@ -44,9 +44,14 @@ def _both_ways(L, shapes, ws, rank, is_avg, seed):
     assert L.tftq_quantize(h, ptrs, addr(table), addr(dev_ptrs), addr(packed), size, dev, stream) == 0
     a, b = packed.clone(), packed.clone()
     assert L.tftq_reduce(h, addr(table), addr(a), size, rank, is_avg, dev, stream) == 0
-    before = torch.cuda.memory_allocated()
+    # nothing is allocated: neither in torch's allocator nor, as far as the driver's count of
+    # free device memory shows, behind its back
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     assert L.tftq_reduce_static(h, addr(b), size, rank, is_avg, dev, stream) == 0
+    torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     # error paths queue nothing
     assert L.tftq_reduce_static(h, addr(b), size - 4, rank, is_avg, dev, stream) == -4
     assert L.tftq_reduce_static(h, addr(b), size, ws, is_avg, dev, stream) == -1
@@ -85,4 +90,90 @@ def test_reduce_static_refuses_tables_beyond_its_array():
     L.tftq_plan_destroy(h)
     h = _plan(L, [(4, 40)] * 2000, 2)  # this one fits
     assert 0 < L.tftq_plan_table_bytes(h) <= 512 * 1024
+    L.tftq_plan_destroy(h)
+
+
+def test_reduce_static_is_busy_for_other_streams_until_its_kernel_has_finished():
+    """All calls on a device share one array.  A second call on the same stream is ordered
+    behind the first; on another stream, while the first call's kernel has not finished, it
+    returns TFTQ_E_BUSY and queues nothing; once the first stream has drained it goes through."""
+    from torchft_amd import _lib
+    L = _lib.load()
+    assert L.tftq_check_device(0) == 0
+    shapes = [(5 + i % 9, 40 + 8 * (i % 7)) for i in range(30)]
+    ws, rank = 2, 1
+    h = _plan(L, shapes, ws)
+    size = L.tftq_plan_output_size(h)
+    nbytes = L.tftq_plan_table_bytes(h)
+    host = (ctypes.c_uint8 * nbytes).from_address(L.tftq_plan_table_host(h))
+    table = torch.frombuffer(host, dtype=torch.uint8).cuda()
+    ts = [torch.randn(s, device="cuda").to(torch.bfloat16) for s in shapes]
+    ptrs = (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    dev_ptrs = torch.empty(len(ts), dtype=torch.int64, device="cuda")
+    packed = torch.empty(size, dtype=torch.uint8, device="cuda")
+    dev = torch.cuda.current_device()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    assert L.tftq_quantize(h, ptrs, p(table), p(dev_ptrs), p(packed), size, dev,
+                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    want = packed.clone()
+    assert L.tftq_reduce(h, p(table), p(want), size, rank, 0, dev,
+                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    a, b, c = packed.clone(), packed.clone(), packed.clone()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        torch.cuda._sleep(int(4.0e8))  # the first call's kernels sit behind this
+    raw1, raw2 = ctypes.c_void_p(s1.cuda_stream), ctypes.c_void_p(s2.cuda_stream)
+    assert L.tftq_reduce_static(h, p(a), size, rank, 0, dev, raw1) == 0
+    assert L.tftq_reduce_static(h, p(b), size, rank, 0, dev, raw1) == 0      # same stream: ordered
+    rc = L.tftq_reduce_static(h, p(c), size, rank, 0, dev, raw2)               # another stream: refused
+    assert rc == -9 and b"still in use" in L.tftq_strerror(rc)
+    s1.synchronize()
+    assert torch.equal(c, packed), "a refused call must not have touched its buffer"
+    assert L.tftq_reduce_static(h, p(c), size, rank, 0, dev, raw2) == 0      # now it goes through
+    torch.cuda.synchronize()
+    for got, name in ((a, "first"), (b, "second, same stream"), (c, "third, other stream")):
+        assert torch.equal(got, want), name
+    L.tftq_plan_destroy(h)
+
+
+def test_reduce_static_under_stream_capture():
+    """A stream capture (global mode) is invalidated by any call that allocates or
+    synchronises: tftq_reduce_static on a long list is recorded in one, and the graph's
+    replays give the bytes of tftq_reduce."""
+    from torchft_amd import _lib
+    L = _lib.load()
+    assert L.tftq_check_device(0) == 0   # looks up the array's address outside the capture
+    shapes = [(4 + i % 11, 24 + 4 * (i % 13)) for i in range(40)]
+    ws, rank = 4, 3
+    h = _plan(L, shapes, ws)
+    size = L.tftq_plan_output_size(h)
+    nbytes = L.tftq_plan_table_bytes(h)
+    host = (ctypes.c_uint8 * nbytes).from_address(L.tftq_plan_table_host(h))
+    table = torch.frombuffer(host, dtype=torch.uint8).cuda()
+    ts = [torch.randn(s, device="cuda").to(torch.bfloat16) for s in shapes]
+    ptrs = (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    dev_ptrs = torch.empty(len(ts), dtype=torch.int64, device="cuda")
+    packed = torch.empty(size, dtype=torch.uint8, device="cuda")
+    dev = torch.cuda.current_device()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    cur = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert L.tftq_quantize(h, ptrs, p(table), p(dev_ptrs), p(packed), size, dev, cur) == 0
+    want = packed.clone()
+    assert L.tftq_reduce(h, p(table), p(want), size, rank, 1, dev, cur) == 0
+    work = packed.clone()
+    torch.cuda.synchronize()
+    cap = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(cap):
+        with torch.cuda.graph(graph, stream=cap):
+            rc = L.tftq_reduce_static(h, p(work), size, rank, 1, dev, ctypes.c_void_p(cap.cuda_stream))
+    assert rc == 0
+    for rep in range(3):
+        work.copy_(packed)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(work, want), f"replay {rep}"
     L.tftq_plan_destroy(h)

@@ -13,7 +13,7 @@ _lib: ctypes.CDLL | None = None
 
 ERR_NAMES = {
     -1: "TFTQ_E_ARG", -2: "TFTQ_E_DTYPE", -3: "TFTQ_E_SHAPE", -4: "TFTQ_E_SIZE",
-    -5: "TFTQ_E_NOMEM", -6: "TFTQ_E_NOTABLE", -7: "TFTQ_E_ARCH", -8: "TFTQ_E_TOOBIG",
+    -5: "TFTQ_E_NOMEM", -6: "TFTQ_E_NOTABLE", -7: "TFTQ_E_ARCH", -8: "TFTQ_E_TOOBIG", -9: "TFTQ_E_BUSY",
 }
 
 # every symbol that include/tftq.h declares: (name, restype, argtypes)

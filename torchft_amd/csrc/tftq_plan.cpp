@@ -37,6 +37,7 @@ extern "C" const char *tftq_strerror(int code)
     case TFTQ_E_NOTABLE: return "a list of more than 16 tensors needs the device table and the pointer buffer";
     case TFTQ_E_ARCH: return "device is not gfx950";
     case TFTQ_E_TOOBIG: return "the list's descriptor table does not fit the library's fixed array";
+    case TFTQ_E_BUSY: return "the library's fixed array is still in use by a call on another stream";
     default: return code > 0 ? "HIP error" : "unknown error";
     }
 }

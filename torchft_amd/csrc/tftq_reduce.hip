@@ -1027,37 +1027,56 @@ extern "C" int tftq_reduce(const tftq_plan *plan, const void *table, void *packe
 // ---------------------------------------------------------------------------
 // Every device the library runs on holds its own copy of this array at its own address.
 // Host code never uses the array's name as an address: it asks the runtime for the address
-// on the current device once (static_table_address) and uses that pointer from then on.
+// on the current device once (static_table_entry) and uses that pointer from then on.
 static __device__ __align__(256) uint8_t static_table[TFTQ_STATIC_TABLE_BYTES];
 
 constexpr int MAX_DEVICES = 64;
-static void *static_table_ptr[MAX_DEVICES];  // per device ordinal; 0 = not looked up yet
+// Per device ordinal: the array's address there, and what guards it.  All calls on a device
+// share the array, so a call must not rewrite it while the kernel of an earlier call, on
+// another stream, may still read it: `done` is recorded behind every reduce kernel, and a
+// call on another stream that finds it unfinished returns TFTQ_E_BUSY instead of racing.
+// Calls on one stream are ordered by the stream.  Calls that a stream capture records run
+// when the graph runs, which this library does not see: they are neither checked nor
+// remembered, and serialising them stays with the caller.
+struct StaticTable {
+    void *ptr = nullptr;        // 0 = not looked up yet
+    hipEvent_t done = nullptr;  // created with the look-up
+    hipStream_t last = nullptr; // stream of the last call that was not captured
+    bool used = false;
+    std::mutex in_call;         // one call at a time writes the array and queues its kernel
+};
+static StaticTable static_tables[MAX_DEVICES];
 static std::mutex static_table_mutex;
 
-// Address of static_table on the device that is current on the calling thread.
-static int static_table_address(void **out)
+// The entry of the device that is current on the calling thread, looked up on first use.
+static int static_table_entry(StaticTable **out)
 {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= MAX_DEVICES) return TFTQ_E_ARG;
+    StaticTable &t = static_tables[dev];
     std::lock_guard<std::mutex> guard(static_table_mutex);
-    if (!static_table_ptr[dev]) {
+    if (!t.ptr) {
         void *p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_table));
         if (e != hipSuccess) return (int)e;
         if (!p) return TFTQ_E_ARG;
-        static_table_ptr[dev] = p;
+        hipEvent_t ev = nullptr;
+        e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+        if (e != hipSuccess) return (int)e;
+        t.done = ev;
+        t.ptr = p;
     }
-    *out = static_table_ptr[dev];
+    *out = &t;
     return 0;
 }
 
 // Set-up for the current device (called by tftq_check_device).
 int tftq_static_table_setup(void)
 {
-    void *p = nullptr;
-    return static_table_address(&p);
+    StaticTable *t = nullptr;
+    return static_table_entry(&t);
 }
 
 extern "C" int tftq_reduce_static(const tftq_plan *plan, void *packed, int64_t packed_bytes, int rank, int is_avg,
@@ -1073,11 +1092,29 @@ extern "C" int tftq_reduce_static(const tftq_plan *plan, void *packed, int64_t p
     if (packed_bytes != plan->output_size) return TFTQ_E_SIZE;  // before anything is queued
     if (rank < 0 || rank >= plan->ws || (!packed && plan->output_size != 0) || ((uintptr_t)packed & 3) != 0)
         return TFTQ_E_ARG;
-    void *table = nullptr;
-    int rc = static_table_address(&table);
+    StaticTable *t = nullptr;
+    int rc = static_table_entry(&t);
     if (rc) return rc;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    hipError_t e = hipStreamIsCapturing(st, &capture);
+    if (e != hipSuccess) return (int)e;
+    const bool captured = capture != hipStreamCaptureStatusNone;
+    std::lock_guard<std::mutex> guard(t->in_call);
+    if (!captured && t->used && t->last != st) {
+        e = hipEventQuery(t->done);
+        if (e == hipErrorNotReady) return TFTQ_E_BUSY;  // an earlier call's kernel, on another stream, may still read the array
+        if (e != hipSuccess) return (int)e;
+    }
     // the whole image every time: the array keeps whatever the last call, of any plan, left there
-    rc = tftq_put_bytes(table, plan->blob.data(), plan->blob.size(), st);
+    rc = tftq_put_bytes(t->ptr, plan->blob.data(), plan->blob.size(), st);
     if (rc) return rc;
-    return reduce_launch(plan, table, packed, packed_bytes, rank, is_avg, st);
+    rc = reduce_launch(plan, t->ptr, packed, packed_bytes, rank, is_avg, st);
+    if (!captured) {
+        // also after a failed launch: the table kernels above are queued and write the array
+        e = hipEventRecord(t->done, st);
+        if (e != hipSuccess) return rc ? rc : (int)e;
+        t->last = st;
+        t->used = true;
+    }
+    return rc;
 }
