@@ -68,6 +68,9 @@ def parse_args():
                          "shape), through torch.distributed's RCCL process group with this process as its only "
                          "rank and through a group of 8 ranks simulated by threads on the one GPU: wall time "
                          "per call against the time of its kernels, and where the host's time goes")
+    ap.add_argument("--footprint", default="3", choices=["2", "3"],
+                    help="with --config ceiling: the configuration whose footprint and product kernels are timed "
+                         "(3: 436 MB of bf16 tensors in 9 tensors; 2: one bf16 tensor of 33.5 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a counter "
@@ -193,25 +196,27 @@ def run_ceilings(args) -> int:
         return {"us": round(mean, 2), "us_min": round(us[0], 2), "bytes": nbytes,
                 "GBs": round(nbytes / mean / 1e3, 1), "frac_of_peak": round(nbytes / mean / 1e3 / HBM_PEAK_GBS, 4)}
 
-    # footprint of benchmark configuration 3: 436 MB of bf16 tensors, 218 MB packed, slots of 27 MB
-    big = 13312 * 32768  # 436 207 616 bytes
-    rows, row_bytes = 6656, 4100  # one slot of 4096-column rows
-    slot = 27292672               # slot size of benchmark configuration 3 (a multiple of 128)
+    # footprint of benchmark configuration 3: 436 MB of bf16 tensors, 218 MB packed, slots of 27 MB;
+    # of configuration 2: 33.5 MB, 16.8 MB, 2.1 MB
+    U = 13312 if args.footprint == "3" else 1024  # chunks of 32 KB
+    big = U * 32768               # 436 207 616 bytes
+    rows, row_bytes = U // 2, 4100  # one slot of 4096-column rows
+    slot = 27292672 if args.footprint == "3" else 2099200  # slot size of the configuration (a multiple of 128)
     bufs = [(torch.empty(big, dtype=torch.uint8, device=dev).random_(),
              torch.empty(big, dtype=torch.uint8, device=dev).random_()) for _ in range(nsets)]
     NT, PLAIN = (1,), (0,)
     BOTH = (0, 1)
     # (label, kind, units, eighths, nt_loads choices, nt_stores choices)
-    kinds = [("read only", 0, 13312, 0, BOTH, PLAIN), ("write only", 1, 13312, 0, PLAIN, BOTH),
-             ("2:1 read:write (quantize, 16-bit tensors)", 2, 13312, 0, BOTH, BOTH),
-             ("1:2 read:write (dequantize, 16-bit tensors)", 3, 13312, 0, BOTH, BOTH),
-             ("4:1 read:write (quantize, fp32 tensors)", 4, 13312, 0, BOTH, BOTH),
-             ("1:4 read:write (dequantize, fp32 tensors)", 5, 13312, 0, BOTH, BOTH),
-             ("2:1 read:write, 4 steps per lane", 11, 26624, 0, NT, NT),
-             ("1:2 read:write, 4 steps per lane", 12, 26624, 0, NT, NT),
-             ("4:1 read:write, 4 steps per lane", 13, 26624, 0, NT, BOTH),
-             ("1:4 read:write, 4 steps per lane", 14, 26624, 0, BOTH, NT),
-             ("8:1 read:write, one contiguous source (reduce, 8 peers)", 6, 6656, 0, BOTH, BOTH),
+    kinds = [("read only", 0, U, 0, BOTH, PLAIN), ("write only", 1, U, 0, PLAIN, BOTH),
+             ("2:1 read:write (quantize, 16-bit tensors)", 2, U, 0, BOTH, BOTH),
+             ("1:2 read:write (dequantize, 16-bit tensors)", 3, U, 0, BOTH, BOTH),
+             ("4:1 read:write (quantize, fp32 tensors)", 4, U, 0, BOTH, BOTH),
+             ("1:4 read:write (dequantize, fp32 tensors)", 5, U, 0, BOTH, BOTH),
+             ("2:1 read:write, 4 steps per lane", 11, 2 * U, 0, NT, NT),
+             ("1:2 read:write, 4 steps per lane", 12, 2 * U, 0, NT, NT),
+             ("4:1 read:write, 4 steps per lane", 13, 2 * U, 0, NT, BOTH),
+             ("1:4 read:write, 4 steps per lane", 14, 2 * U, 0, BOTH, NT),
+             ("8:1 read:write, one contiguous source (reduce, 8 peers)", 6, U // 2, 0, BOTH, BOTH),
              ("reduce's accesses: 8 slots, 4100-byte rows, in place, an eighth of the rows per XCD",
               7, rows, 1, NT, BOTH),
              ("reduce's accesses, rows in workgroup order", 7, rows, 0, NT, BOTH),
@@ -248,7 +253,7 @@ def run_ceilings(args) -> int:
     # the product kernels on benchmark configuration 3, each alone in the same kind of loop
     sets = []
     for k in range(nsets):
-        t = workloads.cfg3(1000 * k + rank, device=dev)
+        t = (workloads.cfg3 if args.footprint == "3" else workloads.cfg2)(1000 * k + rank, device=dev)
         packed = q.fused_quantize_into_fp8(t, ws)
         sets.append({"tensors": t, "recv": packed.clone(), "gathered": packed})
     ab = workloads.algorithmic_bytes(sets[0]["tensors"], ws)
@@ -271,14 +276,16 @@ def run_ceilings(args) -> int:
         c = best(kind)
         product[stage]["ceiling_GBs"] = c["GBs"]
         product[stage]["of_ceiling"] = round(product[stage]["GBs"] / c["GBs"], 4)
-    for stage, kind in (("reduce", 7), ("dequantize", 9)):
+    for stage, kind in (("quantize", 10), ("reduce", 7), ("dequantize", 9)):
         c = best(kind)
         product[stage]["own_accesses_GBs"] = c["GBs"]
         product[stage]["of_own_accesses"] = round(product[stage]["GBs"] / c["GBs"], 4)
     out = {"metric": "streaming ceilings and product kernels, each kernel alone, HBM GB/s on 1 MI355X",
            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-           "config": {"workload": "footprint of benchmark configuration 3 (436 MB of 16-bit tensors, 218 MB "
-                                  f"packed, 8 slots); {nsets} rotating buffer sets"},
+           "config": {"workload": ("footprint of benchmark configuration 3 (436 MB of 16-bit tensors, 218 MB "
+                                   "packed, 8 slots)" if args.footprint == "3" else
+                                   "footprint of configuration 2 (one bf16 tensor of 33.5 MB, 16.8 MB packed, 8 slots)")
+                                  + f"; {nsets} rotating buffer sets"},
            "ceilings": ceilings, "product": product}
     print(json.dumps(out))
     return 0
