@@ -268,7 +268,7 @@ DEV void reduce_row_two_passes(const Seg &s, const KParams &p, int j, int tid, f
                 if (valid) {
                     const u32x4 o = requant16<GDIV>(acc, s2, p);
                     if (doff >= d) {
-                        *(GLOBAL u32x4_a4 *)(orow + 1 + doff) = o;
+                        STORE_CODES(o, (GLOBAL u32x4_a4 *)(orow + 1 + doff));
                     } else {
                         // The vector reaches back into the dwords before this chunk, whose
                         // codes have already been replaced in the own slot: what was
@@ -341,7 +341,7 @@ DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float
     reduce_row_two_passes<GDIV, R_PARKED_CHUNKS>(s, p, j, tid, lds, c, TFTQ_R_DWORDS_WIDE, amax, [&](float s2) {
 #pragma unroll
         for (int u = 0; u < UNITS; u++)
-            *(GLOBAL u32x4_a4 *)(orow + 1 + 4 * (u * TFTQ_WG + tid)) = requant16<GDIV>(acc[u], s2, p);
+            STORE_CODES(requant16<GDIV>(acc[u], s2, p), (GLOBAL u32x4_a4 *)(orow + 1 + 4 * (u * TFTQ_WG + tid)));
     }, parked);
 }
 
