@@ -416,6 +416,35 @@ def test_short_rows_all_team_sizes(q, oracle, ws, op):
     full_check(q, oracle, half, ws, op, [ws // 2])
 
 
+@pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (2, ReduceOp.AVG), (3, ReduceOp.SUM), (4, ReduceOp.AVG),
+                                   (5, ReduceOp.AVG), (7, ReduceOp.SUM), (8, ReduceOp.AVG), (9, ReduceOp.SUM),
+                                   (12, ReduceOp.AVG), (15, ReduceOp.SUM), (16, ReduceOp.AVG), (17, ReduceOp.AVG)])
+def test_rows_of_17_to_64_columns(q, oracle, ws, op):
+    """Every row length from 17 to 64 columns (reduce: pairs of lanes up to 32 columns, teams
+    of 4 lanes above, one vector per lane, in groups of up to 8 and of up to 16 peers; a lane
+    per row in larger groups), row counts that leave the last wavefront and the last workgroup partly or wholly
+    without rows, rows whose scale needs the plain divide next to rows that do not, rows of
+    zeros, and rows in which every peer holds -0."""
+    g = torch.Generator().manual_seed(1700 + ws)
+    rows = [1, ws, ws * 15 + 1, ws * 16, ws * 33 + 2, ws * 70 + 3, ws * 129]
+    shapes = [(rows[c % len(rows)], c) for c in range(17, 65)]
+    peers = []
+    for p in range(ws):
+        ts = []
+        for r, c in shapes:
+            x = torch.randn(r, c, generator=g) * (1 + p % 3)
+            if r > 4:
+                x[1] *= 1e-30
+                x[2] = 0.0
+                x[3] = -0.0
+                x[4, ::2] = -0.0
+            ts.append(x)
+        peers.append(ts)
+    full_check(q, oracle, peers, ws, op, None if ws <= 4 else [0, ws // 2, ws - 1])
+    half = [[t.to(torch.bfloat16) for t in ts] for ts in peers]
+    full_check(q, oracle, half, ws, op, [ws - 1])
+
+
 @pytest.mark.parametrize("ws,op", [(2, ReduceOp.AVG), (8, ReduceOp.SUM), (8, ReduceOp.AVG), (16, ReduceOp.SUM),
                                    (17, ReduceOp.AVG), (32, ReduceOp.SUM), (33, ReduceOp.AVG), (64, ReduceOp.SUM),
                                    (70, ReduceOp.AVG)])

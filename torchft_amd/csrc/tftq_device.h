@@ -113,11 +113,9 @@ DEV float team_bcast(float v, int k)
 template <int TEAM>
 DEV float team_max(float v, float *lds)
 {
-    if (TEAM >= 8) {
-        v = fmaxf(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
-        v = fmaxf(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
-        v = fmaxf(v, dpp_mov<0x141>(v));  // row_half_mirror
-    }
+    if (TEAM >= 2) v = fmaxf(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+    if (TEAM >= 4) v = fmaxf(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+    if (TEAM >= 8) v = fmaxf(v, dpp_mov<0x141>(v));  // row_half_mirror
     if (TEAM >= 16) v = fmaxf(v, dpp_mov<0x140>(v));  // row_mirror: all 16 lanes of a row agree
     if (TEAM >= 32) {
         const float a = bcast_lane(v, 0), b = bcast_lane(v, 16);

@@ -26,6 +26,8 @@ enum : uint8_t {
     K_VEC128 = 14, // two wavefronts per row, 2 rows per workgroup (dequantize only)
     K_VEC256 = 3,  // one workgroup per row (also loops over rows too long for registers)
     K_GEN1 = 4,    // one lane per row, 256 rows per workgroup
+    K_GEN2 = 16,   // 2 lanes per row (reduce only)
+    K_GEN4 = 15,   // 4 lanes per row (reduce only)
     K_GEN8 = 5,    // 8 lanes per row
     K_GEN16 = 9,   // 16 lanes per row (reduce only)
     K_GEN32 = 10,  // 32 lanes per row (reduce only)
@@ -44,6 +46,8 @@ enum : uint8_t {
 TFTQ_HD static inline int tftq_team_of(uint8_t kind)
 {
     switch (kind) {
+    case K_GEN2: return 2;
+    case K_GEN4: return 4;
     case K_VEC8: case K_GEN8: return 8;
     case K_GEN16: case K_VEC16: return 16;
     case K_GEN32: case K_VEC32: return 32;

@@ -122,7 +122,16 @@ static uint8_t pick_reduce_kind(const Seg &s, int ws)
     // one or two 16-byte vectors of codes per lane and peer, four for the longest rows
     const int ndw = s.row_bytes / 4 - 1;
     if (s.n == 1) return K_COL1;
-    if (ndw <= 16) return K_GEN1;  // up to 64 bytes of codes: a lane per row beats a team with idle lanes
+    // 17 to 64 bytes of codes.  A lane per row loads its row with two or four 16-byte loads that
+    // lie a row apart from its neighbours'; a pair of lanes (up to 32 bytes) or a team of 4 with
+    // one vector each covers 32 or 16 neighbouring rows with one load per wavefront and peer
+    // and has every load of its row in flight at once (groups of up to 16 peers).  218 M bf16
+    // elements, 8 peers, a lane per row against the team: 24 columns 81.1 -> 66.7 us, 28: 89.2
+    // -> 64.4, 32: 65.0 -> 64.4, 44: 92.1 -> 68.7, 60: 95.6 -> 64.7, 64: 70.6 -> 65.0; 48 columns
+    // (three whole vectors: a lane per row wastes nothing, the team idles a lane) 67.3 -> 69.4.
+    if (ndw > 8 && ndw <= 16 && ndw != 12 && ws <= 16) return K_GEN4;
+    if (ndw > 4 && ndw <= 8 && ws <= 16) return K_GEN2;
+    if (ndw <= 16) return K_GEN1;  // a lane per row beats a team with idle lanes
     if (ndw <= 32) return K_GEN8;
     if (ndw <= 64) return K_GEN16;
     // Rows that would leave more than a quarter of the next team idle take three vectors per

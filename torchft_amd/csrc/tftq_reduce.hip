@@ -587,6 +587,68 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
     if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
 }
 
+// Rows of up to 16 * TEAM bytes of codes in teams of 2 or 4 lanes: one vector per lane and
+// peer, groups of up to MAXWS (8 or 16) peers, every load of the row in flight at once.  (One
+// lane per row reads such a row with two or four loads that lie a row apart from its
+// neighbours'; here a load instruction of a wavefront covers 32 or 16 neighbouring rows.)
+// Lane l of a team fetches the scales of peers l, l + TEAM, ...: MAXWS / TEAM of them, ahead
+// of the codes: a line that a streaming load has brought in is not kept for a later load.
+// `valid` as in reduce_rows.
+template <int TEAM, int MAXWS, bool GDIV>
+DEV void reduce_rows_narrow(const Seg &s, const KParams &p, int j, int lane, float *lds, bool valid)
+{
+    constexpr int NS = MAXWS / TEAM;  // scales per lane
+    const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
+    const int ws = p.ws;                     // <= MAXWS
+    const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
+    const int doff = min(4 * lane, ndw - 4);  // the last vector ends with the row (see reduce_rows)
+    const u32 padmask = (doff == ndw - 4 && (s.n & 3)) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
+
+    float raw[NS];
+#pragma unroll
+    for (int i = 0; i < NS; i++) raw[i] = as_f(peer_row(p, min(lane + i * TEAM, ws - 1), off)[0]);
+    u32x4 w[MAXWS];
+#pragma unroll
+    for (int k = 0; k < MAXWS; k++)
+        w[k] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k, ws - 1), off) + 1 + doff));
+    __builtin_amdgcn_sched_barrier(0);  // all loads are issued before anything below
+
+    DivCoef c[NS];
+    bool fast = true;
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        c[i] = make_div(raw[i] == 0.0f ? 1.0f : raw[i]);  // padding rows (:419)
+        fast = fast && c[i].fast;
+    }
+    if (__builtin_amdgcn_ballot_w64(!fast) != 0) {
+        if (valid) reduce_row_slow<TEAM, GDIV>(s, p, j, lane, lds);  // some peer needs the plain divide
+        return;
+    }
+
+    float acc[16];  // set by the first peer
+#pragma unroll
+    for (int k = 0; k < MAXWS; k++) {
+        if (k < ws) {
+            const float pr = team_bcast<TEAM>(c[k / TEAM].r, k % TEAM);
+            const float pl = team_bcast<TEAM>(c[k / TEAM].r_lo, k % TEAM);
+            u32x4 v = w[k];
+            v.w &= padmask;
+            if (k == 0) accumulate16<true>(acc, v, pr, pl);
+            else accumulate16<false>(acc, v, pr, pl);
+        }
+    }
+
+    float amax = 0.0f;  // duplicates held by lanes past the row's end do not change it
+#pragma unroll
+    for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[e]));
+    amax = team_max<TEAM>(amax, lds);
+    const float s2 = calc_scale(amax_div<GDIV>(amax, p));  // :340
+    GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
+    const u32x4 o = requant16<GDIV>(acc, s2, p);
+    if (valid && 4 * lane < ndw) STORE_CODES(o, (GLOBAL u32x4_a4 *)(orow + 1 + doff));
+    if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
+}
+
 // One row per team with UNITS >= 2 vectors per lane and peer, as a rolling window over the
 // peers: as soon as a lane has taken vector u of peer k out of its registers, the load of
 // vector u of peer k + 1 is issued into them, so UNITS loads are in flight all the time at
@@ -861,6 +923,12 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
         case K_GEN8:
             if (blk * 32 + (tid >> 3) < s.slice_rows) reduce_row_slow<8, true, true>(s, p, blk * 32 + (tid >> 3), tid & 7, lds);
             break;
+        case K_GEN4:
+            if (blk * 64 + (tid >> 2) < s.slice_rows) reduce_row_slow<4, true, true>(s, p, blk * 64 + (tid >> 2), tid & 3, lds);
+            break;
+        case K_GEN2:
+            if (blk * 128 + (tid >> 1) < s.slice_rows) reduce_row_slow<2, true, true>(s, p, blk * 128 + (tid >> 1), tid & 1, lds);
+            break;
         case K_GEN1:
             if (blk * 256 + tid < s.slice_rows) reduce_row_slow<1, true, true>(s, p, blk * 256 + tid, 0, lds);
             break;
@@ -955,6 +1023,18 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
         if (s.kind[ST_R] == K_GEN32) small(std::integral_constant<int, 32>());
         else if (s.kind[ST_R] == K_GEN16) small(std::integral_constant<int, 16>());
         else small(std::integral_constant<int, 8>());
+        break;
+    }
+    case K_GEN4: {  // one row per team of 4 lanes, groups of up to 16 peers
+        const int j = blk * 64 + (tid >> 2), jc = min(j, s.slice_rows - 1);
+        if (p.ws <= 8) reduce_rows_narrow<4, 8, GDIV>(s, p, jc, tid & 3, lds, j < s.slice_rows);
+        else reduce_rows_narrow<4, 16, GDIV>(s, p, jc, tid & 3, lds, j < s.slice_rows);
+        break;
+    }
+    case K_GEN2: {  // one row per pair of lanes, groups of up to 16 peers
+        const int j = blk * 128 + (tid >> 1), jc = min(j, s.slice_rows - 1);
+        if (p.ws <= 8) reduce_rows_narrow<2, 8, GDIV>(s, p, jc, tid & 1, lds, j < s.slice_rows);
+        else reduce_rows_narrow<2, 16, GDIV>(s, p, jc, tid & 1, lds, j < s.slice_rows);
         break;
     }
     case K_GEN1:  // one lane per row: 1, 2 or 4 vectors of codes per peer
