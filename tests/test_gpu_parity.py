@@ -557,6 +557,22 @@ def test_rows_parked_in_lds(q, oracle):
         full_check(q, oracle, peers, 2, ReduceOp.SUM)
 
 
+@pytest.mark.parametrize("ws,op", [(3, ReduceOp.AVG), (8, ReduceOp.AVG), (9, ReduceOp.SUM), (17, ReduceOp.AVG)])
+def test_reduce_rows_beyond_the_registers(q, oracle, ws, op):
+    """Reduce on rows of more than 32768 columns: 32768 columns of sums stay in registers, the
+    next 16384 are parked in LDS, the rest makes two passes in steps of up to 8 peers whose
+    loads are pipelined.  Lengths at both ends of each range, rows that end inside a vector or
+    a dword, group sizes of one step and of several, a row whose scale needs the plain divide."""
+    g = torch.Generator().manual_seed(4900 + ws)
+    cols = [32772, 36867, 49152, 49153, 49156, 49160, 53248, 53250, 57344, 66001, 131072 + 20]
+    base = [[torch.randn(2 if c < 60000 else 1, c, generator=g).to(torch.bfloat16) * (1 + p) for c in cols]
+            for p in range(3)]
+    base[1][2][0] *= 1e-30
+    base[2][4][1] = 0.0
+    peers = [base[p % 3] for p in range(ws)]
+    full_check(q, oracle, peers, ws, op, [0, ws - 1])
+
+
 def test_long_rows(q, oracle):
     """Rows longer than the register-resident paths hold: 20000 and 70000 columns."""
     g = torch.Generator().manual_seed(21)

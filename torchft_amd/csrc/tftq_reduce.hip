@@ -208,84 +208,137 @@ DEV void reduce_row_slow(const Seg &s, const KParams &p, int j, int lane, float 
 // every row (:318-372), but with 16-byte loads, the fast exact division and the
 // scales read once.  The second pass reads the peer rows again (from the
 // caches if they are still there).
-// The passes cover the dwords from d0 on; the caller has dealt with the dwords
-// before d0, hands in their maximum and stores them in `between`, which runs
-// when the new scale is known and every lane has finished reading for the
+// The passes cover the dwords from d0 on.  The caller deals with the dwords before d0:
+// `middle` runs between the first pass and the row maximum and returns their maximum (it
+// may read the peers' rows, the own slot included: nothing has been stored yet), `between`
+// stores them, when the new scale is known and every lane has finished reading for the
 // first pass.  c: division coefficients of peer min(lane, ws - 1), all fast.
 // PARK: the sums of the first PARK chunks are parked in LDS (parked: PARK * 16 KB) by the
 // first pass and taken from there by the second, which then reads no peer for them.
-template <bool GDIV, int PARK, typename Between>
+// A step is a chunk's vectors of up to 8 peers; the loads of the next step are in flight
+// while the current one is accumulated (53248 bf16 columns, 8 peers: 62.3 us with steps of 4
+// peers one after the other, 56.0 us with steps of 8).
+constexpr int R_STEP_PEERS = 8;
+template <bool GDIV, int PARK, typename Middle, typename Between>
 DEV void reduce_row_two_passes(const Seg &s, const KParams &p, int j, int tid, float *lds, const DivCoef &c,
-                               int d0, float amax, Between between, float *parked = nullptr)
+                               int d0, Middle middle, Between between, float *parked = nullptr)
 {
+    constexpr int CHUNK = 4 * TFTQ_WG;  // dwords
     const int ndw = (s.row_bytes >> 2) - 1;
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
     const int ws = p.ws;  // <= 64 here
     GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
     const u32 tailmask = (s.n & 3) ? (1u << (8 * (s.n & 3))) - 1u : 0xFFFFFFFFu;
-    float s2 = 0.0f;
-#pragma nounroll
-    for (int pass = 0; pass < 2; pass++) {
-#pragma nounroll
-        for (int d = d0; d < ndw; d += 4 * TFTQ_WG) {
-            const bool valid = d + 4 * tid < ndw;
-            const int doff = min(d + 4 * tid, ndw - 4);  // the last vector ends with the row
-            const u32 mask = doff == ndw - 4 ? tailmask : 0xFFFFFFFFu;
-            const int chunk = (d - d0) / (4 * TFTQ_WG);
-            const bool in_lds = PARK > 0 && chunk < PARK;  // same for the whole workgroup
-            float acc[16];
-            if (pass == 1 && in_lds) {
+    const int nchunks = (ndw - d0 + CHUNK - 1) / CHUNK;
+    const int nbatches = (ws + R_STEP_PEERS - 1) / R_STEP_PEERS;  // steps per chunk
+    float amax = 0.0f, s2 = 0.0f;
+
+    struct Step {
+        u32x4 w[R_STEP_PEERS];
+    };
+    // loads of batch `bi` of chunk `ci`
+    auto issue = [&](Step &dst, int ci, int bi) {
+        const int doff = min(d0 + ci * CHUNK + 4 * tid, ndw - 4);  // the last vector ends with the row
 #pragma unroll
-                for (int e = 0; e < 16; e++) acc[e] = parked[(chunk * 16 + e) * TFTQ_WG + tid];
-            } else {
+        for (int b = 0; b < R_STEP_PEERS; b++)
+            dst.w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(bi * R_STEP_PEERS + b, ws - 1), off) + 1 + doff));
+    };
+    // what both passes do with the sums of a chunk
+    auto finish = [&](const float (&acc)[16], int ci, int pass) {
+        const int d = d0 + ci * CHUNK;
+        const int doff = min(d + 4 * tid, ndw - 4);
+        if (pass == 0) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[e]));
+            if (PARK > 0 && ci < PARK) {  // every lane reads back only what it wrote
+#pragma unroll
+                for (int e = 0; e < 16; e++) parked[(ci * 16 + e) * TFTQ_WG + tid] = acc[e];
+            }
+        } else {
+            // the moved-back last vector overlaps its neighbour, which may sit in another
+            // wavefront: nobody stores before everybody has read the own slot's chunk
+            __syncthreads();
+            if (d + 4 * tid < ndw) {
+                const u32x4 o = requant16<GDIV>(acc, s2, p);
+                if (doff >= d) {
+                    STORE_CODES(o, (GLOBAL u32x4_a4 *)(orow + 1 + doff));
+                } else {
+                    // The vector reaches back into the dwords before this chunk, whose
+                    // codes have already been replaced in the own slot: what was
+                    // accumulated for those dwords is meaningless and they are final already.
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (doff + e >= d) orow[1 + doff + e] = o[e];
+                }
+            }
+        }
+    };
+
+    auto run_pass = [&](auto pass_c) {
+        constexpr int pass = decltype(pass_c)::value;
+        float acc[16];
+        // the second pass takes the parked chunks from LDS and loads from the first one behind them
+        const int first = pass == 0 ? 0 : min(PARK, nchunks);
+        if (pass == 1) {
+#pragma nounroll
+            for (int ci = 0; ci < first; ci++) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[e] = parked[(ci * 16 + e) * TFTQ_WG + tid];
+                finish(acc, ci, 1);
+            }
+        }
+        // steps (chunk, batch) in order; ci, bi: the step to consume, ni, nb: the step to issue
+        int ci = first, bi = 0, ni = first, nb = 0;
+        auto advance = [&](int &chunk, int &batch) {
+            if (++batch == nbatches) {
+                batch = 0;
+                ++chunk;
+            }
+        };
+        auto consume = [&](const Step &src) {
+            const u32 mask = min(d0 + ci * CHUNK + 4 * tid, ndw - 4) == ndw - 4 ? tailmask : 0xFFFFFFFFu;
+            if (bi == 0) {
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+            }
+#pragma unroll
+            for (int b = 0; b < R_STEP_PEERS; b++) {
+                const int k = bi * R_STEP_PEERS + b;
+                u32x4 w = src.w[b];
+                w.w &= mask;
+                if (k < ws) accumulate16(acc, w, bcast_lane(c.r, k), bcast_lane(c.r_lo, k));
+            }
+            if (bi == nbatches - 1) finish(acc, ci, pass);
+            advance(ci, bi);
+        };
+        Step A, B;
+        if (ni < nchunks) {
+            issue(A, ni, nb);
+            advance(ni, nb);
+        }
 #pragma nounroll
-                for (int k0 = 0; k0 < ws; k0 += 4) {
-                    u32x4 w[4];
-#pragma unroll
-                    for (int b = 0; b < 4; b++) {
-                        w[b] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(peer_row(p, min(k0 + b, ws - 1), off) + 1 + doff));
-                    }
-#pragma unroll
-                    for (int b = 0; b < 4; b++) {
-                        w[b].w &= mask;
-                        if (k0 + b < ws) accumulate16(acc, w[b], bcast_lane(c.r, k0 + b), bcast_lane(c.r_lo, k0 + b));
-                    }
-                }
+        while (ci < nchunks) {  // A holds the step to consume
+            const bool more = ni < nchunks;
+            if (more) {
+                issue(B, ni, nb);
+                advance(ni, nb);
             }
-            if (pass == 0) {
-#pragma unroll
-                for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[e]));
-                if (in_lds) {  // every lane reads back only what it wrote
-#pragma unroll
-                    for (int e = 0; e < 16; e++) parked[(chunk * 16 + e) * TFTQ_WG + tid] = acc[e];
+            consume(A);
+            if (more) {
+                if (ni < nchunks) {
+                    issue(A, ni, nb);
+                    advance(ni, nb);
                 }
-            } else {
-                // the moved-back last vector overlaps its neighbour, which may sit in another
-                // wavefront: nobody stores before everybody has read the own slot's chunk
-                __syncthreads();
-                if (valid) {
-                    const u32x4 o = requant16<GDIV>(acc, s2, p);
-                    if (doff >= d) {
-                        STORE_CODES(o, (GLOBAL u32x4_a4 *)(orow + 1 + doff));
-                    } else {
-                        // The vector reaches back into the dwords before this chunk, whose
-                        // codes have already been replaced in the own slot: what was
-                        // accumulated for those dwords is meaningless and they are final already.
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (doff + e >= d) orow[1 + doff + e] = o[e];
-                    }
-                }
+                consume(B);
             }
         }
-        if (pass == 0) {
-            amax = team_max<256>(amax, lds);  // every wavefront has read the old scales by now
-            s2 = calc_scale(amax_div<GDIV>(amax, p));
-            between(s2);
-        }
-    }
+    };
+    run_pass(std::integral_constant<int, 0>());
+    amax = fmaxf(amax, middle());
+    amax = team_max<256>(amax, lds);  // every wavefront has read the old scales by now
+    s2 = calc_scale(amax_div<GDIV>(amax, p));
+    between(s2);
+    run_pass(std::integral_constant<int, 1>());
     if (tid == 0) orow[0] = as_u(s2);  // :375
 }
 
@@ -298,14 +351,18 @@ DEV void reduce_row_long(const Seg &s, const KParams &p, int j, int tid, float *
         reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
         return;
     }
-    reduce_row_two_passes<GDIV, 0>(s, p, j, tid, lds, c, 0, 0.0f, [](float) {});
+    reduce_row_two_passes<GDIV, 0>(s, p, j, tid, lds, c, 0, [] { return 0.0f; }, [](float) {});
 }
 
 // Wide kernel, rows of more than 8192 payload dwords: the sums of the first 8192
-// dwords stay in registers (128 per lane), those of the next 3072 are parked in
-// 48 KB of LDS and only the rest of the row makes two passes, so the peers are
-// read 1 + rest / length times instead of twice (53248 columns: 1.15 times).
-constexpr int R_PARKED_CHUNKS = 3;  // chunks of 1024 dwords = 16 KB of sums each
+// dwords stay in registers (128 per lane), those of the next 4096 are parked in
+// 64 KB of LDS and only the rest of the row makes two passes, so the peers are
+// read 1 + rest / length times instead of twice (53248 columns: 1.08 times; with 48 KB of
+// LDS 1.15 times and 57.3 instead of 53.4 us).  Two workgroups of 64 KB fit the 160 KB of a
+// CU, and the registers admit no more than two.
+// The part in registers takes its peers through the rolling window of reduce_rows_roll
+// (53248 columns: 65.4 -> 62.3 us against all vectors of a peer loaded, then summed).
+constexpr int R_PARKED_CHUNKS = 4;  // chunks of 1024 dwords = 16 KB of sums each
 template <bool GDIV>
 DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float *lds, float *parked)
 {
@@ -317,28 +374,56 @@ DEV void reduce_row_hybrid(const Seg &s, const KParams &p, int j, int tid, float
         reduce_row_slow<256, GDIV>(s, p, j, tid, lds);
         return;
     }
-    float acc[UNITS][16];
-#pragma unroll
-    for (int u = 0; u < UNITS; u++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) acc[u][e] = 0.0f;
-#pragma nounroll
-    for (int k = 0; k < ws; k++) {
-        GLOBAL const u32 *pv = peer_row(p, k, off) + 1;
+    // The part of the row behind the registers' makes its first pass first (its loads pipelined in
+    // registers that the sums of the part in front do not hold yet), then the part in front
+    // is summed, then the row maximum is known and both are stored.
+    float acc[UNITS][16];  // set by the first peer
+    auto front = [&]() {
+        // the rolling window of reduce_rows_roll: vector u of the next peer is loaded as soon as
+        // vector u of this one has left its registers
         u32x4 w[UNITS];
+        {
+            GLOBAL const u32 *pv = peer_row(p, 0, off) + 1;
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + 4 * (u * TFTQ_WG + tid)));
-        const float pr = bcast_lane(c.r, k), pl = bcast_lane(c.r_lo, k);
+            for (int u = 0; u < UNITS; u++) w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + 4 * (u * TFTQ_WG + tid)));
+        }
+        {   // the first peer (a group of one reads it a second time and ignores that)
+            const float pr = bcast_lane(c.r, 0), pl = bcast_lane(c.r_lo, 0);
+            GLOBAL const u32 *pv = peer_row(p, min(1, ws - 1), off) + 1;
 #pragma unroll
-        for (int u = 0; u < UNITS; u++) accumulate16(acc[u], w[u], pr, pl);
-    }
-    float amax = 0.0f;
+            for (int u = 0; u < UNITS; u++) {
+                u32x4 x = w[u];
+                asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));
+                w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + 4 * (u * TFTQ_WG + tid)));
+                accumulate16<true>(acc[u], x, pr, pl);
+            }
+        }
+#pragma nounroll
+        for (int k = 1; k + 1 < ws; k++) {
+            const float pr = bcast_lane(c.r, k), pl = bcast_lane(c.r_lo, k);
+            GLOBAL const u32 *pv = peer_row(p, k + 1, off) + 1;
 #pragma unroll
-    for (int u = 0; u < UNITS; u++)
+            for (int u = 0; u < UNITS; u++) {
+                u32x4 x = w[u];
+                asm volatile("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w));  // taken out before the registers are loaded again
+                w[u] = LOAD_STREAM((GLOBAL const u32x4_a4 *)(pv + 4 * (u * TFTQ_WG + tid)));
+                accumulate16(acc[u], x, pr, pl);
+            }
+        }
+        if (ws > 1) {
+            const float pr = bcast_lane(c.r, ws - 1), pl = bcast_lane(c.r_lo, ws - 1);
 #pragma unroll
-        for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+            for (int u = 0; u < UNITS; u++) accumulate16(acc[u], w[u], pr, pl);
+        }
+        float amax = 0.0f;
+#pragma unroll
+        for (int u = 0; u < UNITS; u++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) amax = fmaxf(amax, __builtin_fabsf(acc[u][e]));
+        return amax;
+    };
     GLOBAL u32 *orow = as_global<u32>(p.packed + (int64_t)p.rank * p.slot_size + off);
-    reduce_row_two_passes<GDIV, R_PARKED_CHUNKS>(s, p, j, tid, lds, c, TFTQ_R_DWORDS_WIDE, amax, [&](float s2) {
+    reduce_row_two_passes<GDIV, R_PARKED_CHUNKS>(s, p, j, tid, lds, c, TFTQ_R_DWORDS_WIDE, front, [&](float s2) {
 #pragma unroll
         for (int u = 0; u < UNITS; u++)
             STORE_CODES(requant16<GDIV>(acc[u], s2, p), (GLOBAL u32x4_a4 *)(orow + 1 + 4 * (u * TFTQ_WG + tid)));
@@ -893,7 +978,7 @@ template <bool INLINE, bool GDIV, bool WIDE>
 __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams p, const InlineTable inl)
 {
     __shared__ float lds[16];
-    __shared__ float parked[WIDE ? R_PARKED_CHUNKS * 16 * TFTQ_WG : 1];  // wide kernel: 48 KB (two workgroups per CU fit)
+    __shared__ float parked[WIDE ? R_PARKED_CHUNKS * 16 * TFTQ_WG : 1];  // wide kernel: 64 KB (two workgroups per CU fit)
     Seg s;
     int vb;
     if (!locate<INLINE, ST_R>(p, inl, s, vb)) return;
@@ -1015,7 +1100,7 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
                 if (p.ws <= TEAM) reduce_rows_roll<TEAM, 3, GDIV>(s, p, min(j, s.slice_rows - 1), tid % TEAM, lds, j < s.slice_rows);
                 else if (j < s.slice_rows) reduce_row_slow<TEAM, GDIV>(s, p, j, tid % TEAM, lds);
             } else if (p.ws <= TEAM) {
-                reduce_rows<TEAM, 1, true, GDIV>(s, p, min(j, s.slice_rows - 1), tid % TEAM, lds, j < s.slice_rows);
+                TFTQ_REDUCE_ROWS(TEAM, 1, s, p, min(j, s.slice_rows - 1), tid % TEAM, lds, j < s.slice_rows);
             } else {
                 reduce_row<TEAM, 1, GDIV>(s, p, j, tid % TEAM, lds);
             }
