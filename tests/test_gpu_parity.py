@@ -419,15 +419,16 @@ def test_short_rows_all_team_sizes(q, oracle, ws, op):
 @pytest.mark.parametrize("ws,op", [(1, ReduceOp.SUM), (2, ReduceOp.AVG), (3, ReduceOp.SUM), (4, ReduceOp.AVG),
                                    (5, ReduceOp.AVG), (7, ReduceOp.SUM), (8, ReduceOp.AVG), (9, ReduceOp.SUM),
                                    (12, ReduceOp.AVG), (15, ReduceOp.SUM), (16, ReduceOp.AVG), (17, ReduceOp.AVG)])
-def test_rows_of_17_to_64_columns(q, oracle, ws, op):
-    """Every row length from 17 to 64 columns (reduce: pairs of lanes up to 32 columns, teams
-    of 4 lanes above, one vector per lane, in groups of up to 8 and of up to 16 peers; a lane
-    per row in larger groups), row counts that leave the last wavefront and the last workgroup partly or wholly
+def test_rows_of_13_to_64_columns(q, oracle, ws, op):
+    """Every row length from 13 to 64 columns (reduce: a lane per row up to 16 columns, pairs of
+    lanes up to 32, teams of 4 lanes above, one vector per lane, every peer's vector in flight at
+    once in groups of up to 2, 4, 8 and 16 peers; a lane per row with batches of peers in larger
+    groups), row counts that leave the last wavefront and the last workgroup partly or wholly
     without rows, rows whose scale needs the plain divide next to rows that do not, rows of
     zeros, and rows in which every peer holds -0."""
     g = torch.Generator().manual_seed(1700 + ws)
     rows = [1, ws, ws * 15 + 1, ws * 16, ws * 33 + 2, ws * 70 + 3, ws * 129]
-    shapes = [(rows[c % len(rows)], c) for c in range(17, 65)]
+    shapes = [(rows[c % len(rows)], c) for c in range(13, 65)]
     peers = []
     for p in range(ws):
         ts = []

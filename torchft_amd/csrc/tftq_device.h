@@ -102,6 +102,8 @@ DEV float team_bcast(float v, int k)
 {
     if constexpr (TEAM >= 64) {
         return bcast_lane(v, k);
+    } else if constexpr (TEAM == 1) {
+        return v;
     } else {
         const int base = (int)(threadIdx.x & 63u) & ~(TEAM - 1);
         return __int_as_float(__builtin_amdgcn_ds_bpermute((base + k) << 2, __float_as_int(v)));

@@ -672,8 +672,8 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
     if (valid && lane == 0) orow[0] = as_u(s2);  // :375; all lanes read the old scale before team_max
 }
 
-// Rows of up to 16 * TEAM bytes of codes in teams of 2 or 4 lanes: one vector per lane and
-// peer, groups of up to MAXWS (8 or 16) peers, every load of the row in flight at once.  (One
+// Rows of up to 16 * TEAM bytes of codes in teams of 1, 2 or 4 lanes: one vector per lane and
+// peer, groups of up to MAXWS (2, 4, 8 or 16) peers, every load of the row in flight at once.  (One
 // lane per row reads such a row with two or four loads that lie a row apart from its
 // neighbours'; here a load instruction of a wavefront covers 32 or 16 neighbouring rows.)
 // Lane l of a team fetches the scales of peers l, l + TEAM, ...: MAXWS / TEAM of them, ahead
@@ -682,7 +682,7 @@ DEV void reduce_rows(const Seg &s, const KParams &p, int j, int lane, float *lds
 template <int TEAM, int MAXWS, bool GDIV>
 DEV void reduce_rows_narrow(const Seg &s, const KParams &p, int j, int lane, float *lds, bool valid)
 {
-    constexpr int NS = MAXWS / TEAM;  // scales per lane
+    constexpr int NS = MAXWS > TEAM ? MAXWS / TEAM : 1;  // scales per lane
     const int ndw = (s.row_bytes >> 2) - 1;  // >= 4 here
     const int ws = p.ws;                     // <= MAXWS
     const int64_t off = s.slot_off + (int64_t)j * s.row_bytes;
@@ -974,9 +974,27 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
         else reduce_rows<TEAM, UNITS, true, GDIV>(__VA_ARGS__);                                   \
     } while (0)
 
-template <bool INLINE, bool GDIV, bool WIDE>
-__global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams p, const InlineTable inl)
+// reduce_rows_narrow for a team of TEAM lanes, for the smallest of 2, 4, 8 and 16 peers that
+// holds the group (a variant for more peers loads the last peer again in their place)
+#define TFTQ_REDUCE_NARROW(TEAM, ...)                                             \
+    do {                                                                          \
+        if (p.ws <= 2) reduce_rows_narrow<TEAM, 2, GDIV>(__VA_ARGS__);            \
+        else if (p.ws <= 4) reduce_rows_narrow<TEAM, 4, GDIV>(__VA_ARGS__);       \
+        else if (p.ws <= 8) reduce_rows_narrow<TEAM, 8, GDIV>(__VA_ARGS__);       \
+        else reduce_rows_narrow<TEAM, 16, GDIV>(__VA_ARGS__);                     \
+    } while (0)
+
+// FLAVOUR: R_ALL, every kind of row; R_WIDE, for lists with rows of more than 16384 columns:
+// every kind, twice the registers, half the resident wavefronts; R_LONG, for lists whose rows
+// all run in teams of 64 or 256 lanes (a layer bucket of matrices): only those kinds.  What
+// the compiler makes of one kind's code depends on what else the kernel holds (registers
+// kept across the switch, the order of the blocks): with R_LONG the code for the long rows
+// of such lists is compiled on its own and does not move when another kind's code changes.
+enum { R_ALL = 0, R_WIDE = 1, R_LONG = 2 };
+template <bool INLINE, bool GDIV, int FLAVOUR>
+__global__ __launch_bounds__(TFTQ_WG, FLAVOUR == R_WIDE ? 2 : 4) void k_reduce(const KParams p, const InlineTable inl)
 {
+    constexpr bool WIDE = FLAVOUR == R_WIDE;
     __shared__ float lds[16];
     __shared__ float parked[WIDE ? R_PARKED_CHUNKS * 16 * TFTQ_WG : 1];  // wide kernel: 64 KB (two workgroups per CU fit)
     Seg s;
@@ -994,7 +1012,7 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
     if (GDIV && p.div_mode == 3) {
         // averages over 1024 peers or more, not a power of two: the untuned path with plain divides
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        switch (s.kind[ST_R]) {
+        switch (FLAVOUR == R_LONG ? (s.kind[ST_R] == K_GEN64 ? K_GEN64 : K_GEN256) : s.kind[ST_R]) {
         case K_GEN256: reduce_row_slow<256, true, true>(s, p, blk, tid, lds); break;
         case K_GEN64:
             if (blk * 4 + wave < s.slice_rows) reduce_row_slow<64, true, true>(s, p, blk * 4 + wave, tid & 63, lds);
@@ -1022,7 +1040,8 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
         }
         return;
     }
-    switch (s.kind[ST_R]) {
+    // (R_LONG: one of the two kinds that it is launched for, whatever the table says)
+    switch (FLAVOUR == R_LONG ? (s.kind[ST_R] == K_GEN64 ? K_GEN64 : K_GEN256) : s.kind[ST_R]) {
     case K_GEN256: {  // one workgroup per row, or per 2 or 4 rows when the group is small
         const int rows = tftq_reduce_rows_at_once(K_GEN256, ndw, p.ws);
         const int j = blk * rows;
@@ -1111,19 +1130,20 @@ __global__ __launch_bounds__(TFTQ_WG, WIDE ? 2 : 4) void k_reduce(const KParams 
         break;
     }
     case K_GEN4: {  // one row per team of 4 lanes, groups of up to 16 peers
-        const int j = blk * 64 + (tid >> 2), jc = min(j, s.slice_rows - 1);
-        if (p.ws <= 8) reduce_rows_narrow<4, 8, GDIV>(s, p, jc, tid & 3, lds, j < s.slice_rows);
-        else reduce_rows_narrow<4, 16, GDIV>(s, p, jc, tid & 3, lds, j < s.slice_rows);
+        const int j = blk * 64 + (tid >> 2);
+        TFTQ_REDUCE_NARROW(4, s, p, min(j, s.slice_rows - 1), tid & 3, lds, j < s.slice_rows);
         break;
     }
     case K_GEN2: {  // one row per pair of lanes, groups of up to 16 peers
-        const int j = blk * 128 + (tid >> 1), jc = min(j, s.slice_rows - 1);
-        if (p.ws <= 8) reduce_rows_narrow<2, 8, GDIV>(s, p, jc, tid & 1, lds, j < s.slice_rows);
-        else reduce_rows_narrow<2, 16, GDIV>(s, p, jc, tid & 1, lds, j < s.slice_rows);
+        const int j = blk * 128 + (tid >> 1);
+        TFTQ_REDUCE_NARROW(2, s, p, min(j, s.slice_rows - 1), tid & 1, lds, j < s.slice_rows);
         break;
     }
     case K_GEN1:  // one lane per row: 1, 2 or 4 vectors of codes per peer
-        if (ndw & 3) {  // not whole 16-byte vectors
+        if (ndw == 4 && p.ws <= 16) {  // one whole vector, all peers in flight at once
+            const int j = blk * 256 + tid;
+            TFTQ_REDUCE_NARROW(1, s, p, min(j, s.slice_rows - 1), 0, lds, j < s.slice_rows);
+        } else if (ndw & 3) {  // not whole 16-byte vectors
             if (ndw <= 4) reduce_row<1, 1, GDIV, true>(s, p, blk * 256 + tid, 0, lds);
             else if (ndw <= 8) reduce_row<1, 2, GDIV, true>(s, p, blk * 256 + tid, 0, lds);
             else reduce_row<1, 4, GDIV, true>(s, p, blk * 256 + tid, 0, lds);
@@ -1168,14 +1188,16 @@ static int reduce_launch(const tftq_plan *plan, const void *table, void *packed,
     if (kp.nwg == 0) return 0;
     const unsigned grid = grid_of(kp);
     const bool gdiv = kp.div_mode >= 2;
-#define TFTQ_LAUNCH_R(I, G, W) return launch_kernel(k_reduce<I, G, W>, grid, 0, st, kp, inl)
-    if (plan->wide[ST_R]) {
-        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, true); else TFTQ_LAUNCH_R(false, true, true); }
-        else { if (use_inline) TFTQ_LAUNCH_R(true, false, true); else TFTQ_LAUNCH_R(false, false, true); }
-    } else {
-        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, false); else TFTQ_LAUNCH_R(false, true, false); }
-        else { if (use_inline) TFTQ_LAUNCH_R(true, false, false); else TFTQ_LAUNCH_R(false, false, false); }
-    }
+#define TFTQ_LAUNCH_R(I, G, F) return launch_kernel(k_reduce<I, G, F>, grid, 0, st, kp, inl)
+#define TFTQ_LAUNCH_R_FLAVOUR(F)                                                                        \
+    do {                                                                                                \
+        if (gdiv) { if (use_inline) TFTQ_LAUNCH_R(true, true, F); else TFTQ_LAUNCH_R(false, true, F); } \
+        else { if (use_inline) TFTQ_LAUNCH_R(true, false, F); else TFTQ_LAUNCH_R(false, false, F); }    \
+    } while (0)
+    if (plan->wide[ST_R]) TFTQ_LAUNCH_R_FLAVOUR(R_WIDE);
+    else if (plan->reduce_long_rows) TFTQ_LAUNCH_R_FLAVOUR(R_LONG);
+    else TFTQ_LAUNCH_R_FLAVOUR(R_ALL);
+#undef TFTQ_LAUNCH_R_FLAVOUR
 #undef TFTQ_LAUNCH_R
 }
 
