@@ -262,7 +262,7 @@ struct tftq_plan {
     int64_t max_rows;
     int32_t nwg[3];
     bool wide[3];              // per stage: some row needs the kernel variant with more registers
-    bool reduce_long_rows;     // every row of the list runs in a team of 64 or 256 lanes in reduce (k_reduce's R_LONG)
+    bool reduce_long_rows;     // every row of the list runs in a team of 64 or 256 lanes in reduce or has one column (k_reduce's R_LONG)
     int parked;                // quantize: groups of 5 vectors per lane (20 KB of LDS each, up to 3) that the longest row parks in LDS (rows above TFTQ_Q_VECS_WIDE)
     Dealt dealt[3];            // inline table only
     int32_t dealt_per_xcd[3];  // inline table only: workgroups of the busiest XCD

@@ -380,7 +380,8 @@ extern "C" int tftq_plan_create(int dtype, int n_tensors, const int64_t *shapes,
     for (int i = 0; i < n_tensors; i++) {
         const Seg &s = p->segs[(size_t)i];
         const int nvec = s.n / (16 / p->esz), ndw = s.row_bytes / 4 - 1;
-        if (s.m > 0 && s.kind[ST_R] != K_GEN256 && s.kind[ST_R] != K_GEN64) p->reduce_long_rows = false;
+        if (s.m > 0 && s.kind[ST_R] != K_GEN256 && s.kind[ST_R] != K_GEN64 && s.kind[ST_R] != K_COL1)
+            p->reduce_long_rows = false;
         if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS && s.m > 0) p->wide[ST_Q] = true;
         if (s.kind[ST_Q] == K_VEC256 && nvec > TFTQ_Q_VECS_WIDE && s.m > 0) p->parked = std::max(p->parked, tftq_q_park_groups(nvec));
         if (s.kind[ST_R] == K_GEN256 && ndw > TFTQ_R_DWORDS && s.m > 0 && ws <= 64)

@@ -986,11 +986,13 @@ DEV void reduce_col1(const Seg &s, const KParams &p, int j0, int tid)
 
 // FLAVOUR: R_ALL, every kind of row; R_WIDE, for lists with rows of more than 16384 columns:
 // every kind, twice the registers, half the resident wavefronts; R_LONG, for lists whose rows
-// all run in teams of 64 or 256 lanes (a layer bucket of matrices): only those kinds.  What
+// all run in teams of 64 or 256 lanes or have one column (a layer bucket: matrices, norm
+// weights, biases): only those kinds.  What
 // the compiler makes of one kind's code depends on what else the kernel holds (registers
 // kept across the switch, the order of the blocks): with R_LONG the code for the long rows
 // of such lists is compiled on its own and does not move when another kind's code changes.
 enum { R_ALL = 0, R_WIDE = 1, R_LONG = 2 };
+DEV int long_kind(int kind) { return kind == K_GEN64 ? K_GEN64 : kind == K_COL1 ? K_COL1 : K_GEN256; }
 template <bool INLINE, bool GDIV, int FLAVOUR>
 __global__ __launch_bounds__(TFTQ_WG, FLAVOUR == R_WIDE ? 2 : 4) void k_reduce(const KParams p, const InlineTable inl)
 {
@@ -1012,7 +1014,7 @@ __global__ __launch_bounds__(TFTQ_WG, FLAVOUR == R_WIDE ? 2 : 4) void k_reduce(c
     if (GDIV && p.div_mode == 3) {
         // averages over 1024 peers or more, not a power of two: the untuned path with plain divides
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        switch (FLAVOUR == R_LONG ? (s.kind[ST_R] == K_GEN64 ? K_GEN64 : K_GEN256) : s.kind[ST_R]) {
+        switch (FLAVOUR == R_LONG ? long_kind(s.kind[ST_R]) : s.kind[ST_R]) {
         case K_GEN256: reduce_row_slow<256, true, true>(s, p, blk, tid, lds); break;
         case K_GEN64:
             if (blk * 4 + wave < s.slice_rows) reduce_row_slow<64, true, true>(s, p, blk * 4 + wave, tid & 63, lds);
@@ -1040,8 +1042,8 @@ __global__ __launch_bounds__(TFTQ_WG, FLAVOUR == R_WIDE ? 2 : 4) void k_reduce(c
         }
         return;
     }
-    // (R_LONG: one of the two kinds that it is launched for, whatever the table says)
-    switch (FLAVOUR == R_LONG ? (s.kind[ST_R] == K_GEN64 ? K_GEN64 : K_GEN256) : s.kind[ST_R]) {
+    // (R_LONG: one of the three kinds that it is launched for, whatever the table says)
+    switch (FLAVOUR == R_LONG ? long_kind(s.kind[ST_R]) : s.kind[ST_R]) {
     case K_GEN256: {  // one workgroup per row, or per 2 or 4 rows when the group is small
         const int rows = tftq_reduce_rows_at_once(K_GEN256, ndw, p.ws);
         const int j = blk * rows;
