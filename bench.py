@@ -36,10 +36,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch on benchmark configuration 3 as profiled (profiles/cfg3_bf16_ws8_hbm_traffic.md)
-PROFILED_TRAFFIC = {"quantize": 655472640, "reduce": 247994880, "dequantize": 660084736}
+PROFILED_TRAFFIC = {"quantize": 655474688, "reduce": 248143667, "dequantize": 660078592}
 # mean kernel durations in the step of the same workload by rocprofv3 --kernel-trace, us
 # (profiles/cfg3_bf16_ws8_kernel_trace.md): the cross-check of the event times below
-PROFILED_KERNEL_US = {"quantize": 109.6, "reduce": 44.0, "dequantize": 108.1}
+PROFILED_KERNEL_US = {"quantize": 109.3, "reduce": 43.2, "dequantize": 108.1}
 
 
 def parse_args():
