@@ -1191,6 +1191,53 @@ def test_plan_cache_eviction(q, oracle, monkeypatch):
         same_bytes(got, oracle.fused_quantize_into_fp8(list(ts), ws), "quantize after eviction")
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_group_sizes_and_row_lengths(q, oracle, seed):
+    """Lists of 1 to 20 tensors with a random group size from 1 to 20, SUM or AVG, any of the
+    three dtypes: mostly rows of 1 to 70 columns (a lane, a pair or a team of 4 per row in
+    reduce, on both sides of their group sizes 2, 4, 8 and 16), rows of up to 600 columns, rows
+    at the limits of what reduce keeps in registers and parks in LDS (32768, 49152 columns and
+    their neighbours) and rows of up to 140 000 columns; row counts from one to 200 per rank,
+    rows that take the plain divide, rows of -0."""
+    import random
+    rnd = random.Random(seed)
+    for case in range(14):
+        ws = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 20])
+        op = rnd.choice([ReduceOp.AVG, ReduceOp.SUM])
+        dtype = rnd.choice([torch.bfloat16, torch.float32, torch.float16])
+        shapes = []
+        for _ in range(rnd.choice([1, 3, 12, 20])):
+            kind = rnd.random()
+            if kind < 0.55:
+                c = rnd.randint(1, 70)
+            elif kind < 0.75:
+                c = rnd.randint(65, 600)
+            elif kind < 0.85:
+                c = rnd.choice([32768, 32769, 32772, 49151, 49152, 49153, 49157, 53248]) + rnd.choice([0, 0, 1, 3, 4])
+            else:
+                c = rnd.randint(32769, 140000)
+            r = rnd.choice([1, 2, ws, ws + 1, 3 * ws + 2, 40 * ws + 7, 200 * ws]) if c < 2000 else rnd.choice([1, 2, ws + 1])
+            if r * c * ws > 40_000_000:
+                r = 1
+            shapes.append((r, c))
+        g = torch.Generator().manual_seed(1000 * seed + case)
+        base = []
+        for p in range(min(ws, 3)):
+            ts = []
+            for r, c in shapes:
+                x = torch.randn(r, c, generator=g) * (1 + p)
+                if r > 2 and rnd.random() < 0.3:
+                    x[1] *= 1e-30
+                if r > 3 and rnd.random() < 0.3:
+                    x[2] = -0.0
+                ts.append(x.to(dtype))
+            base.append(ts)
+        peers = [base[p % len(base)] for p in range(ws)]
+        ranks = None if ws <= 3 else sorted({0, rnd.randrange(ws), ws - 1})
+        print(f"case {case}: ws {ws} {op} {dtype} {shapes}", flush=True)
+        full_check(q, oracle, peers, ws, op, ranks)
+
+
 @pytest.mark.parametrize("seed", range(int(os.environ.get("TFTQ_RANDOM_EXTREMES", "12"))))
 def test_random_extremes(q, oracle, seed):
     """Random lists at the far ends: group sizes up to 70, rows of up to 70 003 columns,
